@@ -1,0 +1,90 @@
+"""ctypes binding of libflashmuon_hip.so (the declarations mirror include/flashmuon.h).
+
+There is no fallback: if the library has not been built, or a call returns a non-zero status,
+an exception is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashmuon_hip.so")
+
+# fm_status values (include/flashmuon.h)
+FM_OK = 0
+FM_ERR_ALIAS = 5
+FM_BF16, FM_F16, FM_F32 = 0, 1, 2
+
+_DTYPE_CODE = {torch.bfloat16: FM_BF16, torch.float16: FM_F16, torch.float32: FM_F32}
+
+_vp, _i64, _i32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float,
+                              ctypes.c_size_t)
+
+# name -> (restype, argtypes); one entry per FM_API declaration in include/flashmuon.h
+SIGNATURES = {
+    "fm_status_string": (ctypes.c_char_p, [_i32]),
+    "fm_version": (ctypes.c_char_p, []),
+    "fm_syrk_workspace_bytes": (_sz, [_i32, _i32]),
+    "fm_syrk_bf16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
+    "fm_syrk_poly_bf16": (_i32, [_vp, _i64, _vp, _i64, _i32, _f32, _f32, _vp, _sz, _vp]),
+    "fm_gemm_axpby_bf16": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32, _i32,
+                                  _f32, _vp, _sz, _vp]),
+    "fm_sumsq_workspace_bytes": (_sz, []),
+    "fm_sumsq": (_i32, [_vp, _i32, _i32, _i32, _i64, _vp, _vp, _sz, _vp]),
+    "fm_scale_cast_bf16": (_i32, [_vp, _i32, _i32, _i32, _i64, _vp, _f32, _vp, _i64, _vp, _i64, _vp]),
+    "fm_newtonschulz_workspace_bytes": (_sz, [_i32, _i32]),
+    "fm_newtonschulz_bf16": (_i32, [_vp, _i32, _i32, _i32, _i64, _vp, _i64, _i32, _f32, _f32, _f32,
+                                    _f32, _vp, _sz, _vp]),
+    "fm_momentum_nesterov": (_i32, [_vp, _vp, _i32, _i64, _f32, _f32, _i32, _vp]),
+    "fm_weight_update": (_i32, [_vp, _i32, _vp, _i64, _f32, _f32, _vp]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library once and attach the C signatures."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s is missing: build it with `python -m flash_muon_amd.build` "
+                "(there is no fallback path)" % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class FlashMuonError(RuntimeError):
+    def __init__(self, fn, status):
+        self.status = status
+        msg = load().fm_status_string(status).decode()
+        super().__init__("%s failed with status %d: %s" % (fn, status, msg))
+
+
+def check(fn, status):
+    if status != FM_OK:
+        raise FlashMuonError(fn, status)
+
+
+def dtype_code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s (bfloat16, float16, float32 are supported)" % dtype)
+
+
+def stream_ptr(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def workspace(nbytes, device):
+    """Scratch for one call, taken from torch's caching allocator on the current stream."""
+    if nbytes == 0:
+        return None, 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws, nbytes

@@ -1,0 +1,314 @@
+// HBM-bound kernels of the Muon step for gfx950: sum of squares, normalise + cast (+ transpose),
+// momentum / Nesterov update and the decayed weight update.  All are streaming kernels with
+// 16-byte accesses per lane on the aligned path and a scalar path for everything else.
+#include "fm_internal.h"
+
+namespace fm {
+
+// ---- element access by dtype code -------------------------------------------------------------
+template <int DT> struct Elem;
+template <> struct Elem<0> {  // bf16
+  typedef unsigned short raw;
+  static __device__ __forceinline__ float ld(raw v) { return (float)__builtin_bit_cast(bf16_t, v); }
+  static __device__ __forceinline__ raw st(float f) { return __builtin_bit_cast(raw, (bf16_t)f); }
+};
+template <> struct Elem<1> {  // fp16
+  typedef unsigned short raw;
+  static __device__ __forceinline__ float ld(raw v) { return (float)__builtin_bit_cast(_Float16, v); }
+  static __device__ __forceinline__ raw st(float f) { return __builtin_bit_cast(raw, (_Float16)f); }
+};
+template <> struct Elem<2> {  // fp32
+  typedef float raw;
+  static __device__ __forceinline__ float ld(raw v) { return v; }
+  static __device__ __forceinline__ raw st(float f) { return f; }
+};
+
+// value of an input element after the `.bfloat16()` cast the reference applies first
+template <int DT>
+__device__ __forceinline__ float as_bf16_value(typename Elem<DT>::raw v) {
+  return (float)(bf16_t)Elem<DT>::ld(v);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Block-wide sum with a fixed tree: lanes by xor-shuffle, then waves in index order.
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* red /* NT/64 floats of LDS */) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float s = 0.0f;
+#pragma unroll
+  for (int w = 0; w < NT / 64; ++w) s += red[w];
+  __syncthreads();
+  return s;
+}
+
+// ---- sum of squares -----------------------------------------------------------------------------
+template <int DT, bool FLAT_VEC>
+__global__ __launch_bounds__(256) void sumsq_partial_kernel(const void* Gv, int rows, int cols,
+                                                            int64_t ldg, float* partials) {
+  typedef typename Elem<DT>::raw raw;
+  __shared__ float red[4];
+  const raw* G = reinterpret_cast<const raw*>(Gv);
+  const int64_t n = (int64_t)rows * cols;
+  float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+  if (FLAT_VEC) {
+    // contiguous, 16-byte aligned, n a multiple of the vector width
+    constexpr int V = 16 / sizeof(raw);
+    const int64_t nv = n / V;
+    const uint4* G4 = reinterpret_cast<const uint4*>(Gv);
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += (int64_t)gridDim.x * 256) {
+      union { uint4 v; raw e[V]; } u;
+      u.v = G4[i];
+#pragma unroll
+      for (int e = 0; e < V; e += 4) {
+        float a = as_bf16_value<DT>(u.e[e]), b = as_bf16_value<DT>(u.e[e + 1]);
+        float c = as_bf16_value<DT>(u.e[e + 2]), d = as_bf16_value<DT>(u.e[e + 3]);
+        s0 += a * a; s1 += b * b; s2 += c * c; s3 += d * d;
+      }
+    }
+  } else {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+      int64_t r = i / cols, c = i - r * cols;
+      float a = as_bf16_value<DT>(G[r * ldg + c]);
+      s0 += a * a;
+    }
+  }
+  float s = block_sum<256>((s0 + s1) + (s2 + s3), red);
+  if (threadIdx.x == 0) partials[blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(256) void sumsq_final_kernel(const float* partials, int n, float* out) {
+  __shared__ float red[4];
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < n; i += 256) s += partials[i];
+  s = block_sum<256>(s, red);
+  if (threadIdx.x == 0) out[0] = s;
+}
+
+int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
+                 float* partials, hipStream_t stream) {
+  const int64_t n = (int64_t)rows * cols;
+  const int esz = dtype == 2 ? 4 : 2;
+  const bool flat = (ldg == cols) && ((reinterpret_cast<uintptr_t>(G) & 15) == 0) &&
+                    (n % (16 / esz) == 0);
+  dim3 grid(kSumsqBlocks), block(256);
+#define FM_SUMSQ(DT)                                                                              \
+  if (flat) hipLaunchKernelGGL((sumsq_partial_kernel<DT, true>), grid, block, 0, stream, G, rows, \
+                               cols, ldg, partials);                                              \
+  else hipLaunchKernelGGL((sumsq_partial_kernel<DT, false>), grid, block, 0, stream, G, rows,     \
+                          cols, ldg, partials);
+  if (dtype == 0) { FM_SUMSQ(0) } else if (dtype == 1) { FM_SUMSQ(1) } else { FM_SUMSQ(2) }
+#undef FM_SUMSQ
+  hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(256), 0, stream, (const float*)partials,
+                     kSumsqBlocks, out);
+  return (int)hipGetLastError();
+}
+
+// ---- normalise, cast, transpose -----------------------------------------------------------------
+// One 64x64 tile of G per block: D gets the tile in place, T gets it transposed through LDS.
+template <int DT>
+__global__ __launch_bounds__(256) void scale_cast_kernel(const void* Gv, int rows, int cols,
+                                                         int64_t ldg, const float* sumsq, float eps,
+                                                         unsigned short* D, int64_t ldd,
+                                                         unsigned short* T, int64_t ldt,
+                                                         int g_vec, int d_vec, int t_vec) {
+  typedef typename Elem<DT>::raw raw;
+  constexpr int PITCH = 66;   // u16 per LDS row: 33 dwords, so column reads spread over the banks
+  __shared__ unsigned short tile[64 * PITCH];
+  const raw* G = reinterpret_cast<const raw*>(Gv);
+  const float denom = __builtin_sqrtf(sumsq[0]) + eps;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tid = threadIdx.x;
+  const int ch = tid & 7;   // 8-element chunk along the contiguous dimension
+
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int lr = pass * 32 + (tid >> 3);
+    const int r = r0 + lr, c = c0 + ch * 8;
+    unsigned short o[8];
+    if (r < rows) {
+      const raw* src = G + (int64_t)r * ldg + c;
+      if (g_vec && c + 8 <= cols) {
+        union { uint4 v[sizeof(raw) / 2]; raw e[8]; } u;
+#pragma unroll
+        for (int q = 0; q < (int)sizeof(raw) / 2; ++q) u.v[q] = reinterpret_cast<const uint4*>(src)[q];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = Elem<0>::st(as_bf16_value<DT>(u.e[e]) / denom);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          o[e] = (c + e < cols) ? Elem<0>::st(as_bf16_value<DT>(src[e]) / denom) : (unsigned short)0;
+      }
+      if (D) {
+        unsigned short* dst = D + (int64_t)r * ldd + c;
+        if (d_vec && c + 8 <= cols) {
+          union { uint4 v; unsigned short h[8]; } w;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w.h[e] = o[e];
+          *reinterpret_cast<uint4*>(dst) = w.v;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) if (c + e < cols) dst[e] = o[e];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = 0;
+    }
+    if (T) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[lr * PITCH + ch * 8 + e] = o[e];
+    }
+  }
+  if (!T) return;
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int lc = pass * 32 + (tid >> 3);   // column of G = row of T
+    const int c = c0 + lc, r = r0 + ch * 8;
+    if (c < cols) {
+      unsigned short* dst = T + (int64_t)c * ldt + r;
+      union { uint4 v; unsigned short h[8]; } w;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w.h[e] = tile[(ch * 8 + e) * PITCH + lc];
+      if (t_vec && r + 8 <= rows) {
+        *reinterpret_cast<uint4*>(dst) = w.v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (r + e < rows) dst[e] = w.h[e];
+      }
+    }
+  }
+}
+
+int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
+                      const float* sumsq, float eps, bf16_t* D, int64_t ldd, bf16_t* T, int64_t ldt,
+                      hipStream_t stream) {
+  const int esz = dtype == 2 ? 4 : 2;
+  const int gv = ((reinterpret_cast<uintptr_t>(G) & 15) == 0) && ((ldg * esz) % 16 == 0);
+  const int dv = D && ((reinterpret_cast<uintptr_t>(D) & 15) == 0) && (ldd % 8 == 0);
+  const int tv = T && ((reinterpret_cast<uintptr_t>(T) & 15) == 0) && (ldt % 8 == 0);
+  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64)), block(256);
+  unsigned short* d = reinterpret_cast<unsigned short*>(D);
+  unsigned short* t = reinterpret_cast<unsigned short*>(T);
+  if (dtype == 0)
+    hipLaunchKernelGGL(scale_cast_kernel<0>, grid, block, 0, stream, G, rows, cols, ldg, sumsq, eps, d, ldd, t, ldt, gv, dv, tv);
+  else if (dtype == 1)
+    hipLaunchKernelGGL(scale_cast_kernel<1>, grid, block, 0, stream, G, rows, cols, ldg, sumsq, eps, d, ldd, t, ldt, gv, dv, tv);
+  else
+    hipLaunchKernelGGL(scale_cast_kernel<2>, grid, block, 0, stream, G, rows, cols, ldg, sumsq, eps, d, ldd, t, ldt, gv, dv, tv);
+  return (int)hipGetLastError();
+}
+
+// ---- momentum + Nesterov ------------------------------------------------------------------------
+__device__ __forceinline__ float lerp_torch(float s, float e, float w) {
+  // the two-branch form torch's lerp uses (weights below 0.5 interpolate from the start point)
+  return (__builtin_fabsf(w) < 0.5f) ? s + w * (e - s) : e - (e - s) * (1.0f - w);
+}
+
+template <int DT>
+__device__ __forceinline__ void momentum_one(typename Elem<DT>::raw& g, typename Elem<DT>::raw& b,
+                                             float w_buf, float w_nes, int nesterov) {
+  float gf = Elem<DT>::ld(g), bf = Elem<DT>::ld(b);
+  b = Elem<DT>::st(lerp_torch(bf, gf, w_buf));
+  if (nesterov) g = Elem<DT>::st(lerp_torch(gf, Elem<DT>::ld(b), w_nes));
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void momentum_kernel(void* gv, void* bv, int64_t n, float w_buf,
+                                                       float w_nes, int nesterov, int vec) {
+  typedef typename Elem<DT>::raw raw;
+  constexpr int V = 16 / sizeof(raw);
+  raw* g = reinterpret_cast<raw*>(gv);
+  raw* b = reinterpret_cast<raw*>(bv);
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  int64_t done = 0;
+  if (vec) {
+    const int64_t nv = n / V;
+    uint4* g4 = reinterpret_cast<uint4*>(gv);
+    uint4* b4 = reinterpret_cast<uint4*>(bv);
+    for (int64_t i = t; i < nv; i += stride) {
+      union { uint4 v; raw e[V]; } ug, ub;
+      ug.v = g4[i]; ub.v = b4[i];
+#pragma unroll
+      for (int e = 0; e < V; ++e) momentum_one<DT>(ug.e[e], ub.e[e], w_buf, w_nes, nesterov);
+      b4[i] = ub.v;
+      if (nesterov) g4[i] = ug.v;
+    }
+    done = nv * V;
+  }
+  for (int64_t i = done + t; i < n; i += stride) momentum_one<DT>(g[i], b[i], w_buf, w_nes, nesterov);
+}
+
+static inline unsigned stream_grid(int64_t n_vec) {
+  int64_t blocks = (n_vec + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 8192) blocks = 8192;   // 32 blocks per CU; the loop strides over the rest
+  return (unsigned)blocks;
+}
+
+int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
+                             int nesterov, hipStream_t stream) {
+  const int vec = ((reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(buf) & 15) == 0);
+  const int V = dtype == 2 ? 4 : 8;
+  dim3 grid(stream_grid(n / V + 1)), block(256);
+  if (dtype == 0) hipLaunchKernelGGL(momentum_kernel<0>, grid, block, 0, stream, g, buf, n, w_buf, w_nes, nesterov, vec);
+  else if (dtype == 1) hipLaunchKernelGGL(momentum_kernel<1>, grid, block, 0, stream, g, buf, n, w_buf, w_nes, nesterov, vec);
+  else hipLaunchKernelGGL(momentum_kernel<2>, grid, block, 0, stream, g, buf, n, w_buf, w_nes, nesterov, vec);
+  return (int)hipGetLastError();
+}
+
+// ---- weight update ------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void weight_update_kernel(void* pv, const unsigned short* u,
+                                                            int64_t n, float decay_mul, float alpha,
+                                                            int vec) {
+  typedef typename Elem<DT>::raw raw;
+  raw* p = reinterpret_cast<raw*>(pv);
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  int64_t done = 0;
+  if (vec) {
+    // 8 elements per lane: 16 bytes of u, 16 (or 32) bytes of p
+    const int64_t nv = n / 8;
+    for (int64_t i = t; i < nv; i += stride) {
+      union { uint4 v; unsigned short h[8]; } uu;
+      union { uint4 v[sizeof(raw) / 2]; raw e[8]; } up;
+      uu.v = reinterpret_cast<const uint4*>(u)[i];
+#pragma unroll
+      for (int q = 0; q < (int)sizeof(raw) / 2; ++q) up.v[q] = reinterpret_cast<uint4*>(pv)[i * (sizeof(raw) / 2) + q];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float pf = Elem<DT>::ld(Elem<DT>::st(Elem<DT>::ld(up.e[e]) * decay_mul));
+        up.e[e] = Elem<DT>::st(pf + alpha * Elem<0>::ld(uu.h[e]));
+      }
+#pragma unroll
+      for (int q = 0; q < (int)sizeof(raw) / 2; ++q) reinterpret_cast<uint4*>(pv)[i * (sizeof(raw) / 2) + q] = up.v[q];
+    }
+    done = nv * 8;
+  }
+  for (int64_t i = done + t; i < n; i += stride) {
+    float pf = Elem<DT>::ld(Elem<DT>::st(Elem<DT>::ld(p[i]) * decay_mul));
+    p[i] = Elem<DT>::st(pf + alpha * Elem<0>::ld(u[i]));
+  }
+}
+
+int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float decay_mul,
+                         float alpha, hipStream_t stream) {
+  const int vec = ((reinterpret_cast<uintptr_t>(p) & 15) == 0) && ((reinterpret_cast<uintptr_t>(u) & 15) == 0);
+  dim3 grid(stream_grid(n / 8 + 1)), block(256);
+  const unsigned short* uu = reinterpret_cast<const unsigned short*>(u);
+  if (p_dtype == 0) hipLaunchKernelGGL(weight_update_kernel<0>, grid, block, 0, stream, p, uu, n, decay_mul, alpha, vec);
+  else if (p_dtype == 1) hipLaunchKernelGGL(weight_update_kernel<1>, grid, block, 0, stream, p, uu, n, decay_mul, alpha, vec);
+  else hipLaunchKernelGGL(weight_update_kernel<2>, grid, block, 0, stream, p, uu, n, decay_mul, alpha, vec);
+  return (int)hipGetLastError();
+}
+
+}  // namespace fm

@@ -1,0 +1,233 @@
+// bf16 MFMA contraction for gfx950: acc = A * B^T with both operands k-contiguous ("NT"),
+// fp32 accumulation in 32x32x16 MFMA tiles, LDS double buffering, fused epilogue and an
+// optional mirrored (transposed) second store.  X*X^T, b*A + c*A*A and a*X + P*X are all
+// instances of it (see GemmArgs).
+#include "fm_internal.h"
+
+namespace fm {
+
+constexpr int BK = 64;                 // k extent of one LDS stage: 64 bf16 = 128 bytes per row
+constexpr int ROW_BYTES = BK * 2;
+
+// 16-byte chunk c of LDS row r lives at chunk position c ^ swz(r).  Any 8 consecutive rows get 8
+// distinct positions within a 128-byte bank group and any 16 consecutive rows get 16 distinct
+// positions within 256 bytes, so a ds_read_b128 of one chunk column over 32 rows is conflict free.
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+__device__ __forceinline__ uint32_t lds_off(int row, int chunk) {
+  return (uint32_t)(row * ROW_BYTES + ((chunk ^ swz(row)) << 4));
+}
+
+// Upper-triangular tile index t (row-major over rows i, columns j >= i) -> (i, j).
+__device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
+  float fT = (float)(2 * T + 1);
+  int ii = (int)((fT - __builtin_sqrtf(fT * fT - 8.0f * (float)t)) * 0.5f);
+  if (ii < 0) ii = 0;
+  if (ii > T - 1) ii = T - 1;
+  // S(i) = number of tiles in rows < i
+  while (ii > 0 && (ii * T - (ii * (ii - 1)) / 2) > t) --ii;
+  while (ii + 1 < T && ((ii + 1) * T - ((ii + 1) * ii) / 2) <= t) ++ii;
+  i = ii;
+  j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
+}
+
+template <int ROWS, int NT, bool ALIGNED>
+struct TileLoader {
+  static constexpr int N = ROWS * 8 / NT;   // 16-byte chunks per thread
+  static_assert(ROWS * 8 % NT == 0, "tile rows must divide over the threads");
+  const bf16_t* ptr[N];   // row base + chunk offset, per chunk
+  uint32_t soff[N];       // swizzled LDS byte offset, per chunk
+  int kch[N];             // k offset of the chunk inside a stage
+
+  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int row0, int nrows, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int idx = tid + i * NT;
+      int row = idx >> 3, ch = idx & 7;
+      int grow = row0 + row;
+      if (grow > nrows - 1) grow = nrows - 1;   // rows past the end repeat the last row; never stored
+      ptr[i] = base + (int64_t)grow * ld + ch * 8;
+      soff[i] = lds_off(row, ch);
+      kch[i] = ch * 8;
+    }
+  }
+
+  __device__ __forceinline__ void load(uint4 (&r)[N], int k0, int K) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int k = k0 + kch[i];
+      if (ALIGNED) {
+        if (k < K) r[i] = *reinterpret_cast<const uint4*>(ptr[i] + k0);
+        else r[i] = make_uint4(0, 0, 0, 0);
+      } else {
+        union { uint4 v; unsigned short h[8]; } u;
+        const unsigned short* s = reinterpret_cast<const unsigned short*>(ptr[i] + k0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) u.h[e] = (k + e < K) ? s[e] : (unsigned short)0;
+        r[i] = u.v;
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(unsigned char* lds, const uint4 (&r)[N]) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) *reinterpret_cast<uint4*>(lds + soff[i]) = r[i];
+  }
+};
+
+__device__ __forceinline__ unsigned short f2bf(float v) {
+  return __builtin_bit_cast(unsigned short, (bf16_t)v);
+}
+__device__ __forceinline__ float bf2f(bf16_t v) { return (float)v; }
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArgs p) {
+  constexpr int NT = 64 * WAVES_M * WAVES_N;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+
+  __shared__ __align__(16) unsigned char smem[2 * STAGE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  int ti, tj;
+  if (p.symmetric) {
+    tri_decode((int)blockIdx.x, p.tiles_m, ti, tj);
+  } else {
+    ti = (int)blockIdx.x / p.tiles_n;
+    tj = (int)blockIdx.x % p.tiles_n;
+  }
+  const int m0 = ti * BM, n0 = tj * BN;
+
+  TileLoader<BM, NT, ALIGNED> la;
+  TileLoader<BN, NT, ALIGNED> lb;
+  la.init(p.A, p.lda, m0, p.Ma, tid);
+  lb.init(p.B, p.ldb, n0, p.Nb, tid);
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // per-lane fragment addresses: row = lane % 32 of each 32-row block, k half = lane / 32
+  uint32_t a_off[TM], b_off[TN];
+  int a_sw[TM], b_sw[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    int row = wm * WM + i * 32 + (lane & 31);
+    a_off[i] = (uint32_t)(row * ROW_BYTES);
+    a_sw[i] = swz(row);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    int row = wn * WN + j * 32 + (lane & 31);
+    b_off[j] = (uint32_t)(A_BYTES + row * ROW_BYTES);
+    b_sw[j] = swz(row);
+  }
+  const int khalf = lane >> 5;
+
+  const int nk = (p.Kc + BK - 1) / BK;
+  uint4 ra[TileLoader<BM, NT, ALIGNED>::N], rb[TileLoader<BN, NT, ALIGNED>::N];
+
+  la.load(ra, 0, p.Kc);
+  lb.load(rb, 0, p.Kc);
+  la.store(smem, ra);
+  lb.store(smem + A_BYTES, rb);
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    unsigned char* cur = smem + (kt & 1) * STAGE;
+    unsigned char* nxt = smem + ((kt + 1) & 1) * STAGE;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      la.load(ra, (kt + 1) * BK, p.Kc);
+      lb.load(rb, (kt + 1) * BK, p.Kc);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8_t fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        fa[i] = *reinterpret_cast<const bf16x8_t*>(cur + a_off[i] + (((ks * 2 + khalf) ^ a_sw[i]) << 4));
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        fb[j] = *reinterpret_cast<const bf16x8_t*>(cur + b_off[j] + (((ks * 2 + khalf) ^ b_sw[j]) << 4));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      la.store(nxt, ra);
+      lb.store(nxt + A_BYTES, rb);
+    }
+    __syncthreads();
+  }
+
+  // Epilogue.  In the 32x32 accumulator, register r of lane l holds
+  // row 8*(r/4) + 4*(l/32) + r%4, column l%32 of the MFMA tile.
+  const bool diag = p.symmetric && (ti == tj);
+  const bool has_e = p.E != nullptr;
+  unsigned short* C = reinterpret_cast<unsigned short*>(p.C);
+  unsigned short* C2 = reinterpret_cast<unsigned short*>(p.C2);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < p.Ma && col < p.Nb) {
+          float v = acc[i][j][r];
+          if (has_e) v = p.alpha * bf2f(p.E[(int64_t)row * p.lde + col]) + p.beta * v;
+          unsigned short h = f2bf(v);
+          // On a diagonal tile only the elements on or above the diagonal are kept, and the
+          // strictly-upper ones are mirrored, so the two triangles come from the same register.
+          if (!diag || col >= row) {
+            if (C) C[(int64_t)row * p.c_rs + (int64_t)col * p.c_cs] = h;
+          }
+          if (C2 && (!p.symmetric || (diag ? col > row : true))) {
+            C2[(int64_t)col * p.c2_rs + (int64_t)row * p.c2_cs] = h;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+static int launch_cfg(GemmArgs a, bool aligned, hipStream_t stream) {
+  a.tiles_m = (a.Ma + BM - 1) / BM;
+  a.tiles_n = (a.Nb + BN - 1) / BN;
+  a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;
+  dim3 grid((unsigned)a.num_tiles), block(64 * WAVES_M * WAVES_N);
+  if (aligned)
+    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true>), grid, block, 0, stream, a);
+  else
+    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false>), grid, block, 0, stream, a);
+  return (int)hipGetLastError();
+}
+
+int launch_gemm_nt(GemmArgs a, hipStream_t stream) {
+  const bool aligned = (a.lda % 8 == 0) && (a.ldb % 8 == 0) && (a.Kc % 8 == 0) &&
+                       ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0) &&
+                       ((reinterpret_cast<uintptr_t>(a.B) & 15) == 0);
+  // Large outputs take 256x256 tiles (8 waves, 128x64 per wave); small ones take 128x128 tiles
+  // (4 waves, 64x64 per wave) so that more workgroups exist than the chip has CUs.
+  const int64_t big_tiles = (int64_t)((a.Ma + 255) / 256) * ((a.Nb + 255) / 256);
+  const int64_t work_tiles = a.symmetric ? (big_tiles + (a.Ma + 255) / 256) / 2 : big_tiles;
+  if (work_tiles >= 256) return launch_cfg<256, 256, 2, 4>(a, aligned, stream);
+  return launch_cfg<128, 128, 2, 2>(a, aligned, stream);
+}
+
+}  // namespace fm

@@ -1,0 +1,48 @@
+// Internal declarations shared by the translation units of libflashmuon_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+namespace fm {
+
+typedef __bf16 bf16_t;
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+// Arguments of the one NT contraction every GEMM-shaped kernel here is an instance of:
+//     acc[i][j] = sum_k A[i][k] * B[j][k]            (A: Ma x Kc, B: Nb x Kc, k contiguous)
+//     v         = E ? alpha * E[i][j] + beta * acc : acc
+//     C [i*c_rs  + j*c_cs ] = bf16(v)                (if C  != nullptr)
+//     C2[j*c2_rs + i*c2_cs] = bf16(v)                (if C2 != nullptr; the mirrored copy)
+// With `symmetric` set, A == B, only tiles on or above the diagonal are computed and C2 == C.
+struct GemmArgs {
+  const bf16_t* A;  int64_t lda;
+  const bf16_t* B;  int64_t ldb;
+  const bf16_t* E;  int64_t lde;
+  bf16_t* C;  int64_t c_rs, c_cs;
+  bf16_t* C2; int64_t c2_rs, c2_cs;
+  int Ma, Nb, Kc;
+  float alpha, beta;
+  int symmetric;
+  int tiles_m, tiles_n;   // number of block tiles along each output dimension
+  int num_tiles;          // tiles actually computed (triangular count when symmetric)
+};
+
+// Enqueue the contraction described by `args` on `stream`.  Returns a hipError_t value.
+int launch_gemm_nt(GemmArgs args, hipStream_t stream);
+
+int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
+                 float* partials, hipStream_t stream);
+int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
+                      const float* sumsq, float eps, bf16_t* D, int64_t ldd, bf16_t* T, int64_t ldt,
+                      hipStream_t stream);
+int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
+                             int nesterov, hipStream_t stream);
+int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float decay_mul,
+                         float alpha, hipStream_t stream);
+
+constexpr int kSumsqBlocks = 1024;   // partial sums written by the first reduction stage
+
+}  // namespace fm

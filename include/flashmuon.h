@@ -1,0 +1,148 @@
+/*
+ * flashmuon.h -- C ABI of libflashmuon_hip.so, the gfx950 (MI355X) kernel library behind
+ * matmul_transpose / matmul_transpose_assign / fast_newtonschulz / Muon.step.
+ *
+ * The reference (nil0x9/flash-muon) has no FFI: its device boundary is a Triton JIT launch
+ * (flash_muon/matmul_transpose_triton.py:91-101) and torch eager ops (flash_muon/muon.py:23-29,
+ * 87-89, 99-100).  Each entry point below names the reference lines it replaces.
+ *
+ * Conventions, common to every entry point:
+ *   - plain C types only; every pointer is device memory owned by the caller;
+ *   - leading dimensions and strides are in ELEMENTS, not bytes;
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued on it and the call returns
+ *     without synchronising; nothing is allocated or freed;
+ *   - the return value is an fm_status; 0 is success; bad arguments are reported before any
+ *     launch; asynchronous device faults surface at the caller's next synchronisation;
+ *   - `ws`/`ws_bytes` is caller-provided scratch of at least the size the matching
+ *     *_workspace_bytes() function returns (it may be NULL when that size is 0).
+ *   - the library is stateless and re-entrant; two calls that share a workspace must be ordered
+ *     on one stream.
+ */
+#ifndef FLASHMUON_H
+#define FLASHMUON_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* fm_stream_t; /* hipStream_t */
+
+/* every entry point is exported; everything else in the library has hidden visibility */
+#define FM_API __attribute__((visibility("default")))
+
+enum fm_status {
+  FM_OK = 0,
+  FM_ERR_NULL = 1,        /* a required pointer is NULL */
+  FM_ERR_SHAPE = 2,       /* a dimension is negative, zero where forbidden, or inconsistent */
+  FM_ERR_STRIDE = 3,      /* a leading dimension is smaller than the row it must hold */
+  FM_ERR_DTYPE = 4,       /* dtype code not one of FM_BF16 / FM_F16 / FM_F32 */
+  FM_ERR_ALIAS = 5,       /* an output overlaps an input it must not overlap */
+  FM_ERR_WORKSPACE = 6,   /* ws is NULL or ws_bytes too small */
+  FM_ERR_LAUNCH = 7,      /* hipLaunchKernel reported an error */
+  FM_ERR_ALIGN = 8        /* a pointer is not aligned to its element size */
+};
+
+enum fm_dtype { FM_BF16 = 0, FM_F16 = 1, FM_F32 = 2 };
+
+/* Human-readable text for a status code (static storage). */
+FM_API const char* fm_status_string(int status);
+
+/* Library version, "major.minor.patch". */
+FM_API const char* fm_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Y = X * X^T, X is M x K bf16 (row stride ldx, unit column stride), Y is M x M bf16 with
+ * arbitrary strides (ldy_row, ldy_col).  Only upper-triangular tiles are computed; every
+ * off-diagonal element is written twice from the same register, so Y == Y^T bit for bit.
+ * fp32 accumulation, one round-to-nearest-even to bf16.
+ * Replaces mmt_kernel + its launch: flash_muon/matmul_transpose_triton.py:20-75, 90-101.
+ */
+FM_API size_t fm_syrk_workspace_bytes(int M, int K);
+FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
+                 int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * P = b*A + c*(A*A) for a SYMMETRIC M x M bf16 matrix A (row stride lda).  Same triangular
+ * schedule and dual store as fm_syrk_bf16; the polynomial is evaluated on the fp32 accumulator
+ * and rounded to bf16 once.  P must not overlap A.
+ * Replaces the second symmetric product and the three elementwise ops after it:
+ * flash_muon/muon.py:27-28.
+ */
+FM_API int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, float b, float c,
+                      void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Xout = a*X + P*X for P (M x M, row stride ldp) and X (M x K, row stride ldx).  The
+ * contraction runs over the rows of X, so the kernel reads X through its transpose
+ * XT (K x M, row stride ldxt), which the caller supplies (fm_scale_cast_bf16 and this function
+ * both produce it).  Either output may be NULL, not both: Xout is M x K (row stride ldo), XoutT
+ * is its transpose K x M (row stride ldot), written from the same registers.
+ * No output may overlap an input.
+ * Replaces flash_muon/muon.py:29 (`X = a * X + B @ X`: one GEMM and two elementwise ops).
+ */
+FM_API int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt,
+                       const void* X, int64_t ldx, void* Xout, int64_t ldo,
+                       void* XoutT, int64_t ldot, int M, int K, float a,
+                       void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * out[0] = sum over the rows x cols matrix G (row stride ldg) of bf16(G[i,j])^2, in fp32,
+ * with a fixed reduction tree (bit-reproducible run to run).  ws needs fm_sumsq_workspace_bytes().
+ * Replaces the reduction inside `X.norm(dim=(-2,-1))`: flash_muon/muon.py:15, 23.
+ */
+FM_API size_t fm_sumsq_workspace_bytes(void);
+FM_API int fm_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
+             void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * D = bf16(G) / (sqrt(sumsq[0]) + eps) and T = D^T.  G is rows x cols of `dtype` (row stride
+ * ldg); D is rows x cols bf16 (row stride ldd); T is cols x rows bf16 (row stride ldt).  Either
+ * output may be NULL, not both.
+ * Replaces the cast, the transposed view, the division and the `.contiguous()` copy of it:
+ * flash_muon/muon.py:15-17, 23 and flash_muon/matmul_transpose_triton.py:88.
+ */
+FM_API int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int64_t ldg,
+                       const float* sumsq, float eps, void* D, int64_t ldd, void* T, int64_t ldt,
+                       fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * The whole quintic Newton-Schulz orthogonalisation of one matrix: G is rows x cols of `dtype`
+ * (row stride ldg), out is rows x cols bf16 (row stride ldout).  Runs fm_sumsq,
+ * fm_scale_cast_bf16 and `steps` x (fm_syrk_bf16, fm_syrk_poly_bf16, fm_gemm_axpby_bf16) on
+ * `stream`, iterating on the wide orientation (M = min(rows, cols)).  steps == 0 returns the
+ * normalised input.  out must not overlap G.
+ * Replaces fast_newtonschulz: flash_muon/muon.py:6-33.
+ */
+FM_API size_t fm_newtonschulz_workspace_bytes(int rows, int cols);
+FM_API int fm_newtonschulz_bf16(const void* G, int dtype, int rows, int cols, int64_t ldg,
+                         void* out, int64_t ldout, int steps, float a, float b, float c, float eps,
+                         void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * In place, elementwise over n elements of `dtype`:
+ *     buf <- lerp(buf, g, w_buf)         (the reference passes w_buf = 1 - momentum)
+ *     g   <- lerp(g, buf, w_nes)         (w_nes = momentum; only when nesterov != 0,
+ *                                         otherwise g is left alone)
+ * lerp(s, e, w) is s + w*(e - s) for |w| < 0.5 and e - (e - s)*(1 - w) otherwise, the form
+ * torch's lerp_ uses.  Each line is computed in fp32 and rounded once to `dtype`, and the second
+ * line reads the ROUNDED buf, as two successive torch lerp_ calls do.
+ * Replaces flash_muon/muon.py:99-100.
+ */
+FM_API int fm_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
+                         int nesterov, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * In place over n elements: p <- round(p * decay_mul) ; p <- round(p + alpha * u), with u bf16
+ * and p of p_dtype; two roundings, as torch's mul_ followed by add_(alpha=) produce.
+ * Replaces flash_muon/muon.py:87-89.
+ */
+FM_API int fm_weight_update(void* p, int p_dtype, const void* u_bf16, int64_t n, float decay_mul,
+                     float alpha, fm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHMUON_H */

@@ -1,0 +1,22 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def lib():
+    """The loaded C-ABI library; built first only if no built library is present."""
+    from flash_muon_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from flash_muon_amd import build
+        build.build(verbose=False)
+    return _lib.load()

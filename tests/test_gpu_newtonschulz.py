@@ -1,0 +1,101 @@
+"""GPU parity of fast_newtonschulz against the fp32 CPU oracle.
+
+Tolerance: Frobenius-relative error <= 1e-2 per Newton-Schulz step, each step started from the
+oracle's state cast to bf16, and <= 1e-2 for the free-running result after the default five
+steps on gradient-like inputs."""
+import pytest
+import torch
+
+from flash_muon_amd import fast_newtonschulz, synthetic
+from oracle import oracle
+from tests import gpu_util
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = 1e-2
+
+
+@pytest.mark.parametrize("rows,cols,rank,seed", [(256, 1024, 8, 3), (512, 512, 16, 4), (1024, 384, 8, 5), (200, 333, 4, 6)])
+def test_per_step_resynchronised(lib, rows, cols, rank, seed):
+    G = synthetic.gradient_like_bf16(rows, cols, rank, seed)
+    _, states = oracle.newtonschulz(G, 5, trace=True)          # wide orientation, fp32
+    for s in range(5):
+        Xin = states[s].bfloat16()
+        ref = oracle.ns_step(Xin.float())
+        Xo, XoT, A, P = gpu_util.ns_step(lib, Xin.to(DEV), oracle.NS_COEFFS)
+        err = oracle.rel_fro(Xo, ref)
+        print("step %d: rel_fro %.3e" % (s + 1, err), flush=True)
+        assert err < TOL
+        assert torch.equal(A, A.T) and torch.equal(P, P.T)
+        assert torch.equal(XoT, Xo.T.contiguous())
+
+
+@pytest.mark.parametrize("rows,cols,rank,seed", [(256, 1024, 8, 3), (512, 512, 16, 4), (1024, 384, 8, 5),
+                                                 (200, 333, 4, 6), (1, 7, 1, 7), (64, 64, 4, 8)])
+def test_free_running_five_steps(rows, cols, rank, seed):
+    G = synthetic.gradient_like_bf16(rows, cols, rank, seed)
+    ref = oracle.newtonschulz(G, 5)
+    got = fast_newtonschulz(G.to(DEV), 5)
+    assert got.dtype == torch.bfloat16 and got.shape == G.shape
+    err = oracle.rel_fro(got, ref)
+    print("free-running 5 steps %dx%d: rel_fro %.3e" % (rows, cols, err), flush=True)
+    assert err < TOL
+
+
+@pytest.mark.parametrize("steps", [0, 1, 2, 3])
+def test_step_counts(steps):
+    G = synthetic.gradient_like_bf16(128, 320, 4, 21)
+    ref = oracle.newtonschulz(G, steps)
+    got = fast_newtonschulz(G.to(DEV), steps)
+    assert oracle.rel_fro(got, ref) < TOL
+    if steps == 0:
+        assert abs(float(got.float().norm()) - 1.0) < 5e-3
+
+
+def test_transpose_invariance_bitwise():
+    G = synthetic.gradient_like_bf16(192, 448, 4, 22).to(DEV)
+    wide = fast_newtonschulz(G, 5)
+    tall = fast_newtonschulz(G.T.contiguous(), 5)
+    assert torch.equal(wide, tall.T)
+    view = fast_newtonschulz(G.T, 5)                    # transposed view, no copy
+    assert torch.equal(view, tall)
+
+
+def test_diagonal_closed_form():
+    sig = torch.tensor([1.0, 0.5, 0.25, 0.125, 0.0625])
+    a, b, c = oracle.NS_COEFFS
+    s = (sig / sig.norm()).double()
+    for _ in range(5):
+        s = a * s + b * s ** 3 + c * s ** 5
+    got = fast_newtonschulz(torch.diag(sig).to(DEV), 5).cpu().double()
+    assert (torch.diagonal(got) - s).abs().max() < 2e-2
+    assert (got - torch.diag(torch.diagonal(got))).abs().max() == 0
+
+
+def test_input_dtypes_and_scale_invariance():
+    G = synthetic.gradient_like_bf16(160, 288, 4, 23)
+    base = fast_newtonschulz(G.to(DEV), 5)
+    assert torch.equal(fast_newtonschulz(G.float().to(DEV), 5), base)       # same values after the bf16 cast
+    assert torch.equal(fast_newtonschulz(G.double().to(DEV), 5), base)
+    scaled = fast_newtonschulz((G * 8).to(DEV), 5)                           # power of two: same mantissas
+    assert oracle.rel_fro(scaled, base.float()) < 1e-2
+    h = fast_newtonschulz(G.half().to(DEV), 5)
+    assert oracle.rel_fro(h, oracle.newtonschulz(G.half(), 5)) < TOL
+
+
+def test_zero_and_padded_inputs():
+    z = fast_newtonschulz(torch.zeros(32, 48, device=DEV), 5)
+    assert torch.equal(z.cpu(), torch.zeros(32, 48, dtype=torch.bfloat16))
+    G = synthetic.gradient_like_bf16(96, 200, 4, 24)
+    pad = torch.zeros(96, 256, dtype=torch.bfloat16, device=DEV)
+    pad[:, :200] = G.to(DEV)
+    assert torch.equal(fast_newtonschulz(pad[:, :200], 5), fast_newtonschulz(G.to(DEV), 5))
+    assert fast_newtonschulz(torch.zeros(0, 8, device=DEV)).shape == (0, 8)
+
+
+def test_singular_values_land_in_band():
+    G = synthetic.gradient_like_bf16(512, 2048, 8, 25)
+    out = fast_newtonschulz(G.to(DEV), 5).float().cpu()
+    sv = torch.linalg.svdvals(out)
+    # the leading singular values (the spike and the bulk above ~1e-3 of the norm) end near 1
+    assert sv[0] < 1.3 and sv[:8].min() > 0.5
