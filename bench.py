@@ -1,0 +1,152 @@
+#!/usr/bin/env python3
+"""Benchmark of the flash-muon hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+A step is one matmul_transpose call on the 8192 x 8192 bf16 input of the square sweep (seed 8192),
+inputs resident in HBM.  Protocol of the reference's benchmark.py:49-79: W warm-up calls, then K
+calls bracketed by device events.  One JSON line is printed; `value` is useful TFLOP/s
+(K*M*(M+1) flop per call), `roofline` prices the same kernel against the dense bf16 MFMA peak,
+`cpu_baseline` is torch's fp32 X @ X.T on the host cores of the same machine.  `extras` holds the
+other timings of the path: vendor GEMM X @ X.T on the same GPU, fast_newtonschulz(5) on 8192^2
+and 4096 x 16384, and Muon.step on Llama-7B shapes.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+DIM = 8192
+
+
+def _time_gpu(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps   # ms per call
+
+
+def _cpu_baseline(X, torch):
+    """torch fp32 X @ X.T on the host (the reference's own baseline, benchmark.py:20-21)."""
+    from oracle import oracle
+    M, K = X.shape
+    t0 = time.perf_counter()
+    oracle.xxt(X)                       # warm-up, also tells us how long one call takes
+    first = time.perf_counter() - t0
+    reps = 3 if first < 8.0 else 1
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        oracle.xxt(X)
+    dt = (time.perf_counter() - t0) / reps
+    from flash_muon_amd import synthetic
+    return {"value": synthetic.syrk_useful_flop(M, K) / dt / 1e12, "unit": "TFLOP/s (useful)",
+            "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "torch CPU fp32 X@X.T on the full %dx%d input, 1 warm-up + %d reps, %.2f s each; "
+                      "os.cpu_count()=%d" % (M, K, reps, dt, os.cpu_count())}
+
+
+def _extras(Xd, steps, warmup, torch):
+    from flash_muon_amd import Muon, fast_newtonschulz, synthetic
+    ex = {}
+    # vendor GEMM for the same product, both BLAS back ends torch can select
+    for name, pref in (("rocblas", "cublas"), ("hipblaslt", "cublaslt")):
+        try:
+            torch.backends.cuda.preferred_blas_library(pref)
+            ex["torch_xxt_%s_ms" % name] = _time_gpu(lambda: torch.matmul(Xd, Xd.T), steps, warmup, torch)
+        except Exception as e:   # report, never hide
+            ex["torch_xxt_%s_ms" % name] = "failed: %s" % e
+    torch.backends.cuda.preferred_blas_library("default")
+    # fast_newtonschulz(5)
+    for rows, cols, rank, seed in ((8192, 8192, 16, 4), (4096, 16384, 8, 3)):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        G = (1e-3 * torch.randn(rows, cols, generator=g, device="cuda", dtype=torch.float32))
+        G = (G / G.norm()).bfloat16()
+        ms = _time_gpu(lambda: fast_newtonschulz(G, 5), 10, 3, torch)
+        fl = synthetic.ns_useful_flop(rows, cols, 5)
+        ex["ns5_%dx%d_ms" % (rows, cols)] = ms
+        ex["ns5_%dx%d_useful_tflops" % (rows, cols)] = fl / ms / 1e9
+        del G
+    # Muon.step on Llama-7B shapes: 32 layers x (4 x 4096^2, 2 x 11008x4096, 1 x 4096x11008)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    params = []
+    for layer in range(32):
+        for (r, c) in synthetic.LLAMA7B_LAYER_SHAPES:
+            p = torch.nn.Parameter((0.02 * torch.randn(r, c, generator=g, device="cuda", dtype=torch.float32)).bfloat16())
+            p.grad = (1e-3 * torch.randn(r, c, generator=g, device="cuda", dtype=torch.float32)).bfloat16()
+            params.append(p)
+    opt = Muon(params, lr=0.02, momentum=0.95, nesterov=True, rank=0, world_size=1)
+    ms = _time_gpu(opt.step, 3, 1, torch)
+    fl = sum(synthetic.ns_useful_flop(r, c, 5) for (r, c) in synthetic.LLAMA7B_LAYER_SHAPES) * 32
+    ex["muon_step_llama7b_ms"] = ms
+    ex["muon_step_llama7b_useful_tflops"] = fl / ms / 1e9
+    ex["muon_step_llama7b_frac_of_peak"] = fl / ms / 1e9 / PEAK_BF16_TFLOPS
+    return ex
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=25)
+    ap.add_argument("--no-extras", action="store_true", help="skip vendor GEMM, Newton-Schulz and Muon.step timings")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the path is built and measured on a single MI355X "
+                 "(Muon's cross-rank gather is out of scope); run with --gpus 1")
+
+    import torch
+    from flash_muon_amd import _lib, matmul_transpose_assign, synthetic
+    if not os.path.exists(_lib.LIB_PATH):
+        from flash_muon_amd import build
+        build.build()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+
+    X = synthetic.gaussian_bf16(DIM, DIM, DIM)
+    Xd = X.cuda()
+    Y = torch.empty(DIM, DIM, dtype=torch.bfloat16, device="cuda")
+    torch.cuda.empty_cache()
+    ms = _time_gpu(lambda: matmul_transpose_assign(Xd, Y), args.steps, args.warmup, torch)
+    assert torch.equal(Y, Y.T), "output is not symmetric"
+
+    useful = synthetic.syrk_useful_flop(DIM, DIM)
+    tflops = useful / ms / 1e9
+    line = {
+        "metric": "matmul_transpose useful TFLOP/s at 8192x8192 bf16",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "matmul_transpose square sweep, dim=8192, bf16 N(0,1), seed 8192",
+                   "M": DIM, "K": DIM},
+        "effective_tflops": 2.0 * DIM * DIM * DIM / ms / 1e9,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None},
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = _cpu_baseline(X, torch)
+    if not args.no_extras:
+        ex = _extras(Xd, args.steps, args.warmup, torch)
+        for k in ("torch_xxt_rocblas_ms", "torch_xxt_hipblaslt_ms"):
+            if isinstance(ex.get(k), float):
+                ex[k.replace("_ms", "_speedup")] = ex[k] / ms
+        line["extras"] = ex
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

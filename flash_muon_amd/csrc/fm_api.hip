@@ -25,7 +25,7 @@ inline int hip_status(int hip_err) { return hip_err == 0 ? FM_OK : FM_ERR_LAUNCH
 
 // workspace of fm_newtonschulz_bf16, carved in this order
 struct NsLayout {
-  size_t sumsq, partials, x[2], xt[2], a, p, gemm, total;
+  size_t sumsq, partials, pdiag, x[2], xt[2], a, p, gemm, total;
 };
 NsLayout ns_layout(int rows, int cols) {
   const size_t M = (size_t)(rows < cols ? rows : cols), K = (size_t)(rows < cols ? cols : rows);
@@ -34,6 +34,7 @@ NsLayout ns_layout(int rows, int cols) {
   auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
   l.sumsq = take(sizeof(float));
   l.partials = take(kSumsqBlocks * sizeof(float));
+  l.pdiag = take(M * sizeof(float));
   for (int i = 0; i < 2; ++i) { l.x[i] = take(M * K * 2); l.xt[i] = take(M * K * 2); }
   l.a = take(M * M * 2);
   l.p = take(M * M * 2);
@@ -89,26 +90,31 @@ int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t l
 }
 
 int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, float b, float c,
-                      void* ws, size_t ws_bytes, fm_stream_t stream) {
+                      float* diag_out, void* ws, size_t ws_bytes, fm_stream_t stream) {
   (void)ws; (void)ws_bytes;
   if (M < 0) return FM_ERR_SHAPE;
   if (M == 0) return FM_OK;
   if (!A || !P) return FM_ERR_NULL;
   if (lda < M || ldp < M) return FM_ERR_STRIDE;
-  if (misaligned(A, 2) || misaligned(P, 2)) return FM_ERR_ALIGN;
+  if (misaligned(A, 2) || misaligned(P, 2) || misaligned(diag_out, 4)) return FM_ERR_ALIGN;
   if (overlaps(mat_range(A, M, M, lda, 2), mat_range(P, M, M, ldp, 2))) return FM_ERR_ALIAS;
+  if (diag_out && (overlaps(mat_range(diag_out, 1, M, M, 4), mat_range(A, M, M, lda, 2)) ||
+                   overlaps(mat_range(diag_out, 1, M, M, 4), mat_range(P, M, M, ldp, 2))))
+    return FM_ERR_ALIAS;
   GemmArgs a = {};
   a.A = a.B = a.E = static_cast<const bf16_t*>(A); a.lda = a.ldb = a.lde = lda;
   a.C = a.C2 = static_cast<bf16_t*>(P);
   a.c_rs = a.c2_rs = ldp; a.c_cs = a.c2_cs = 1;
   a.Ma = a.Nb = a.Kc = M;
   a.alpha = b; a.beta = c; a.symmetric = 1;
+  a.diag_out = diag_out;
   return hip_status(launch_gemm_nt(a, static_cast<hipStream_t>(stream)));
 }
 
 int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt, const void* X,
                        int64_t ldx, void* Xout, int64_t ldo, void* XoutT, int64_t ldot, int M, int K,
-                       float alpha, void* ws, size_t ws_bytes, fm_stream_t stream) {
+                       float alpha, const float* row_alpha, void* ws, size_t ws_bytes,
+                       fm_stream_t stream) {
   (void)ws; (void)ws_bytes;
   if (M < 0 || K < 0) return FM_ERR_SHAPE;
   if (M == 0 || K == 0) return FM_OK;
@@ -117,7 +123,7 @@ int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt,
   if (ldp < M || ldxt < M || ldx < K) return FM_ERR_STRIDE;
   if ((Xout && ldo < K) || (XoutT && ldot < M)) return FM_ERR_STRIDE;
   if (misaligned(P, 2) || misaligned(XT, 2) || misaligned(X, 2) || misaligned(Xout, 2) ||
-      misaligned(XoutT, 2))
+      misaligned(XoutT, 2) || misaligned(row_alpha, 4))
     return FM_ERR_ALIGN;
   const Range in[3] = {mat_range(P, M, M, ldp, 2), mat_range(XT, K, M, ldxt, 2),
                        mat_range(X, M, K, ldx, 2)};
@@ -135,6 +141,7 @@ int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt,
   a.C2 = static_cast<bf16_t*>(XoutT); a.c2_rs = ldot; a.c2_cs = 1;
   a.Ma = M; a.Nb = K; a.Kc = M;
   a.alpha = alpha; a.beta = 1.0f; a.symmetric = 0;
+  a.row_alpha = row_alpha;
   return hip_status(launch_gemm_nt(a, static_cast<hipStream_t>(stream)));
 }
 
@@ -213,20 +220,21 @@ int fm_newtonschulz_bf16(const void* G, int dtype, int rows, int cols, int64_t l
 
   void* A = w + l.a;
   void* P = w + l.p;
+  float* pdiag = reinterpret_cast<float*>(w + l.pdiag);   // diagonal of P, kept in fp32
   for (int s = 0; s < steps; ++s) {
     const bool last = s + 1 == steps;
     st = fm_syrk_bf16(X, K, A, M, 1, M, K, gws, gws_bytes, stream);
     if (st) return st;
-    st = fm_syrk_poly_bf16(A, M, P, M, M, b, c, gws, gws_bytes, stream);
+    st = fm_syrk_poly_bf16(A, M, P, M, M, b, c, pdiag, gws, gws_bytes, stream);
     if (st) return st;
     void* Xn = w + l.x[(s + 1) & 1];
     void* XTn = w + l.xt[(s + 1) & 1];
     if (!last)
-      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, Xn, K, XTn, M, M, K, a, gws, gws_bytes, stream);
+      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, Xn, K, XTn, M, M, K, a, pdiag, gws, gws_bytes, stream);
     else if (!tall)   // the result has G's shape: X itself
-      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, out, ldout, nullptr, 0, M, K, a, gws, gws_bytes, stream);
+      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, out, ldout, nullptr, 0, M, K, a, pdiag, gws, gws_bytes, stream);
     else              // or its transpose
-      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, nullptr, 0, out, ldout, M, K, a, gws, gws_bytes, stream);
+      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, nullptr, 0, out, ldout, M, K, a, pdiag, gws, gws_bytes, stream);
     if (st) return st;
     X = Xn; XT = XTn;
   }

@@ -189,7 +189,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
         const int row = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (row < p.Ma && col < p.Nb) {
           float v = acc[i][j][r];
-          if (has_e) v = p.alpha * bf2f(p.E[(int64_t)row * p.lde + col]) + p.beta * v;
+          if (has_e) {
+            const float al = p.row_alpha ? p.alpha + p.row_alpha[row] : p.alpha;
+            v = al * bf2f(p.E[(int64_t)row * p.lde + col]) + p.beta * v;
+          }
+          if (p.diag_out && row == col) {
+            p.diag_out[row] = v;
+            v = 0.0f;
+          }
           unsigned short h = f2bf(v);
           // On a diagonal tile only the elements on or above the diagonal are kept, and the
           // strictly-upper ones are mirrored, so the two triangles come from the same register.

@@ -13,7 +13,8 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
 // Arguments of the one NT contraction every GEMM-shaped kernel here is an instance of:
 //     acc[i][j] = sum_k A[i][k] * B[j][k]            (A: Ma x Kc, B: Nb x Kc, k contiguous)
-//     v         = E ? alpha * E[i][j] + beta * acc : acc
+//     v         = E ? (alpha + row_alpha[i]) * E[i][j] + beta * acc : acc   (row_alpha optional)
+//     if diag_out and i == j:  diag_out[i] = v (fp32) and v = 0
 //     C [i*c_rs  + j*c_cs ] = bf16(v)                (if C  != nullptr)
 //     C2[j*c2_rs + i*c2_cs] = bf16(v)                (if C2 != nullptr; the mirrored copy)
 // With `symmetric` set, A == B, only tiles on or above the diagonal are computed and C2 == C.
@@ -25,6 +26,8 @@ struct GemmArgs {
   bf16_t* C2; int64_t c2_rs, c2_cs;
   int Ma, Nb, Kc;
   float alpha, beta;
+  const float* row_alpha;   // optional per-row addition to alpha
+  float* diag_out;          // optional fp32 copy of the diagonal, which is then stored as zero
   int symmetric;
   int tiles_m, tiles_n;   // number of block tiles along each output dimension
   int num_tiles;          // tiles actually computed (triangular count when symmetric)

@@ -68,11 +68,16 @@ FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, in
  * P = b*A + c*(A*A) for a SYMMETRIC M x M bf16 matrix A (row stride lda).  Same triangular
  * schedule and dual store as fm_syrk_bf16; the polynomial is evaluated on the fp32 accumulator
  * and rounded to bf16 once.  P must not overlap A.
+ * If diag_out is not NULL it receives the M diagonal values of the polynomial in fp32 and the
+ * diagonal of P is written as zero: the diagonal carries most of P's magnitude near convergence
+ * (about -2.7 where the off-diagonal entries are O(1/sqrt(M))), so keeping it out of bf16 removes
+ * the largest rounding error of a Newton-Schulz step.  fm_gemm_axpby_bf16 takes it back as
+ * row_alpha.
  * Replaces the second symmetric product and the three elementwise ops after it:
  * flash_muon/muon.py:27-28.
  */
 FM_API int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, float b, float c,
-                      void* ws, size_t ws_bytes, fm_stream_t stream);
+                      float* diag_out, void* ws, size_t ws_bytes, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Xout = a*X + P*X for P (M x M, row stride ldp) and X (M x K, row stride ldx).  The
@@ -80,13 +85,15 @@ FM_API int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, i
  * XT (K x M, row stride ldxt), which the caller supplies (fm_scale_cast_bf16 and this function
  * both produce it).  Either output may be NULL, not both: Xout is M x K (row stride ldo), XoutT
  * is its transpose K x M (row stride ldot), written from the same registers.
+ * If row_alpha is not NULL (M floats), row i uses a + row_alpha[i] in place of a, i.e. the
+ * kernel computes a*X + (P + diag(row_alpha))*X with the diagonal term in fp32.
  * No output may overlap an input.
  * Replaces flash_muon/muon.py:29 (`X = a * X + B @ X`: one GEMM and two elementwise ops).
  */
 FM_API int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt,
                        const void* X, int64_t ldx, void* Xout, int64_t ldo,
                        void* XoutT, int64_t ldot, int M, int K, float a,
-                       void* ws, size_t ws_bytes, fm_stream_t stream);
+                       const float* row_alpha, void* ws, size_t ws_bytes, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * out[0] = sum over the rows x cols matrix G (row stride ldg) of bf16(G[i,j])^2, in fp32,

@@ -24,17 +24,20 @@ def syrk(lib, X, Y=None):
     return Y
 
 
-def syrk_poly(lib, A, b, c):
+def syrk_poly(lib, A, b, c, split_diag=False):
+    """P = b*A + c*A*A; with split_diag returns (P with a zero diagonal, fp32 diagonal)."""
     M = A.size(0)
     P = torch.empty(M, M, dtype=torch.bfloat16, device=A.device)
+    d = torch.empty(M, dtype=torch.float32, device=A.device) if split_diag else None
     ws = _ws(lib.fm_syrk_workspace_bytes(M, M), A.device)
     st = lib.fm_syrk_poly_bf16(A.data_ptr(), A.stride(0), P.data_ptr(), P.stride(0), M, b, c,
+                               d.data_ptr() if split_diag else None,
                                ws.data_ptr(), ws.numel(), _stream(A))
     _lib.check("fm_syrk_poly_bf16", st)
-    return P
+    return (P, d) if split_diag else P
 
 
-def gemm_axpby(lib, P, X, a, want_x=True, want_xt=True, XT=None):
+def gemm_axpby(lib, P, X, a, want_x=True, want_xt=True, XT=None, row_alpha=None):
     M, K = X.shape
     if XT is None:
         XT = X.T.contiguous()
@@ -45,7 +48,8 @@ def gemm_axpby(lib, P, X, a, want_x=True, want_xt=True, XT=None):
                                 X.data_ptr(), X.stride(0),
                                 Xo.data_ptr() if want_x else None, Xo.stride(0) if want_x else 0,
                                 XoT.data_ptr() if want_xt else None, XoT.stride(0) if want_xt else 0,
-                                M, K, a, ws.data_ptr(), ws.numel(), _stream(X))
+                                M, K, a, row_alpha.data_ptr() if row_alpha is not None else None,
+                                ws.data_ptr(), ws.numel(), _stream(X))
     _lib.check("fm_gemm_axpby_bf16", st)
     return Xo, XoT
 
@@ -75,6 +79,6 @@ def ns_step(lib, X, coeffs):
     """One Newton-Schulz step on a bf16 device matrix X (M x K, M <= K) through the three kernels."""
     a, b, c = coeffs
     A = syrk(lib, X)
-    P = syrk_poly(lib, A, b, c)
-    Xo, XoT = gemm_axpby(lib, P, X, a)
+    P, d = syrk_poly(lib, A, b, c, split_diag=True)
+    Xo, XoT = gemm_axpby(lib, P, X, a, row_alpha=d)
     return Xo, XoT, A, P

@@ -59,12 +59,12 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.fm_syrk_bf16(X, 8, Y, 8, 1, -1, 8, None, 0, None) == 2              # shape
     assert lib.fm_syrk_bf16(ctypes.c_void_p(0x1001), 8, Y, 8, 1, 8, 8, None, 0, None) == 8   # alignment
     assert lib.fm_syrk_bf16(X, 8, Y, 8, 1, 0, 8, None, 0, None) == 0               # empty: nothing to do
-    assert lib.fm_syrk_poly_bf16(X, 8, X, 8, 8, 1.0, 1.0, None, 0, None) == 5      # P aliases A
+    assert lib.fm_syrk_poly_bf16(X, 8, X, 8, 8, 1.0, 1.0, None, None, 0, None) == 5      # P aliases A
     # Xout overlapping X is rejected: every output tile reads a whole column block of X
     assert lib.fm_gemm_axpby_bf16(X, 8, Y, 8, ctypes.c_void_p(0x400000), 16, ctypes.c_void_p(0x400000), 16,
-                                  None, 0, 8, 16, 1.0, None, 0, None) == 5
+                                  None, 0, 8, 16, 1.0, None, None, 0, None) == 5
     assert lib.fm_gemm_axpby_bf16(X, 8, Y, 8, ctypes.c_void_p(0x400000), 16, None, 0, None, 0,
-                                  8, 16, 1.0, None, 0, None) == 1                  # no output at all
+                                  8, 16, 1.0, None, None, 0, None) == 1            # no output at all
     assert lib.fm_sumsq(X, 7, 4, 4, 4, Y, Y, 4096, None) == 4                      # dtype
     assert lib.fm_sumsq(X, 0, 4, 4, 4, Y, None, 0, None) == 6                      # workspace
     assert lib.fm_newtonschulz_bf16(X, 0, 8, 8, 8, Y, 8, 5, 1.0, 1.0, 1.0, 1e-7, None, 0, None) == 6

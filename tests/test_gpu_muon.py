@@ -36,7 +36,7 @@ def test_first_and_second_step_against_oracle():
     opt = Muon(params, lr=LR, momentum=MU, rank=0, world_size=1)
     assert opt.step() is None
     ref_p, ref_g, ref_b, ref_u = oracle.muon_step(ps, gs, [None] * len(ps), LR, WD, MU, True, 5)
-    for q, g0, rp, rg, rb in zip(params, gs, ref_p, ref_g, ref_b):
+    for i, (q, g0, rp, rg, rb) in enumerate(zip(params, gs, ref_p, ref_g, ref_b)):
         st = opt.state[q]
         assert set(st.keys()) == {"momentum_buffer"}
         # closed form of the first step: buf = (1-mu) g, grad <- (1-mu^2) g, each rounded once
@@ -46,7 +46,6 @@ def test_first_and_second_step_against_oracle():
             oracle.rel_fro(st["momentum_buffer"], (1 - MU) * g0.float()) < 3e-3
         assert oracle.rel_fro(q.data, rp) < 3e-3
         # the move itself: lr * (update of O(1/sqrt(cols)) entries), seen through p's bf16 rounding
-        i = params.index(q)
         delta_ref = rp - (1 - LR * WD) * ps[i].float()
         delta_got = q.data.cpu().float() - (1 - LR * WD) * ps[i].float()
         assert oracle.rel_fro(delta_got, delta_ref) < 0.15
@@ -111,7 +110,7 @@ def test_conv_filter_param_and_fp32_param():
     assert oracle.rel_fro(q.grad, ref_g[0]) < 1e-6
     delta_got = q.data.cpu() - (1 - LR * WD) * ps[0]
     delta_ref = ref_p[0] - (1 - LR * WD) * ps[0]
-    assert oracle.rel_fro(delta_got, delta_ref) < 1e-2       # the update itself, at NS tolerance
+    assert oracle.rel_fro(delta_got, delta_ref) < 2e-2       # the update itself, at NS tolerance (80 rows)
 
 
 def test_groups_state_dict_and_missing_grad():

@@ -72,12 +72,30 @@ def test_axpby_gaussian(lib):
     assert oracle.rel_fro(Xo, ref) < 3e-3
 
 
+def test_split_diagonal_roundtrip(lib):
+    """The fp32 diagonal that fm_syrk_poly_bf16 hands out and fm_gemm_axpby_bf16 takes back."""
+    M, K = 200, 328
+    A = _int_sym(M, 91, -1, 1)
+    Ai = A.double().round().long()
+    full = (Ai + 2 * (Ai @ Ai))
+    P, d = gpu_util.syrk_poly(lib, A.to(DEV), 1.0, 2.0, split_diag=True)
+    assert torch.equal(d.cpu().long(), torch.diagonal(full))
+    assert (torch.diagonal(P) == 0).all()
+    off = full - torch.diag(torch.diagonal(full))
+    assert torch.equal(P.cpu(), off.float().bfloat16())
+    g = torch.Generator().manual_seed(92)
+    X = torch.randint(-1, 2, (M, K), generator=g).float().bfloat16()
+    want = (3 * X.double() + full.double() @ X.double()).float().bfloat16()
+    Xo, XoT = gpu_util.gemm_axpby(lib, P, X.to(DEV), 3.0, row_alpha=d)
+    assert torch.equal(Xo.cpu(), want) and torch.equal(XoT.cpu(), want.T)
+
+
 def test_axpby_rejects_aliasing(lib):
     X = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
     P = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
     XT = torch.zeros(128, 64, dtype=torch.bfloat16, device=DEV)
     st = lib.fm_gemm_axpby_bf16(P.data_ptr(), 64, XT.data_ptr(), 64, X.data_ptr(), 128, X.data_ptr(), 128,
-                                None, 0, 64, 128, 1.0, None, 0, None)
+                                None, 0, 64, 128, 1.0, None, None, 0, None)
     assert st == 5
 
 
