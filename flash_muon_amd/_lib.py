@@ -24,7 +24,7 @@ _vp, _i64, _i32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, cty
 SIGNATURES = {
     "fm_status_string": (ctypes.c_char_p, [_i32]),
     "fm_version": (ctypes.c_char_p, []),
-    "fm_syrk_workspace_bytes": (_sz, [_i32, _i32]),
+    "fm_gemm_workspace_bytes": (_sz, [_i32, _i32]),
     "fm_syrk_bf16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
     "fm_syrk_poly_bf16": (_i32, [_vp, _i64, _vp, _i64, _i32, _f32, _f32, _vp, _vp, _sz, _vp]),
     "fm_gemm_axpby_bf16": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32, _i32,

@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJDIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libflashmuon_hip.so")
-SOURCES = ["fm_gemm.hip", "fm_elementwise.hip", "fm_api.hip"]
+SOURCES = ["fm_gemm.hip", "fm_gemm_fast.hip", "fm_elementwise.hip", "fm_api.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -22,6 +22,8 @@ inline bool misaligned(const void* p, int esz) { return (reinterpret_cast<uintpt
 inline int dtype_size(int dt) { return dt == FM_F32 ? 4 : 2; }
 inline bool bad_dtype(int dt) { return dt != FM_BF16 && dt != FM_F16 && dt != FM_F32; }
 inline int hip_status(int hip_err) { return hip_err == 0 ? FM_OK : FM_ERR_LAUNCH; }
+// a workspace is only used when it is 256-byte aligned; otherwise the call runs without one
+inline void* usable_ws(void* ws) { return (reinterpret_cast<uintptr_t>(ws) % 256 == 0) ? ws : nullptr; }
 
 // workspace of fm_newtonschulz_bf16, carved in this order
 struct NsLayout {
@@ -38,7 +40,7 @@ NsLayout ns_layout(int rows, int cols) {
   for (int i = 0; i < 2; ++i) { l.x[i] = take(M * K * 2); l.xt[i] = take(M * K * 2); }
   l.a = take(M * M * 2);
   l.p = take(M * M * 2);
-  l.gemm = take(fm_syrk_workspace_bytes((int)M, (int)(K > M ? K : M)));
+  l.gemm = take(fm_gemm_workspace_bytes((int)M, (int)K));
   l.total = off;
   return l;
 }
@@ -64,14 +66,13 @@ const char* fm_status_string(int status) {
 
 const char* fm_version(void) { return "0.1.0"; }
 
-size_t fm_syrk_workspace_bytes(int M, int K) {
-  (void)M; (void)K;
-  return 0;
+size_t fm_gemm_workspace_bytes(int rows_out, int cols_out) {
+  if (rows_out <= 0 || cols_out <= 0) return 0;
+  return gemm_fast_workspace_bytes(rows_out, cols_out, false);
 }
 
 int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
                  void* ws, size_t ws_bytes, fm_stream_t stream) {
-  (void)ws; (void)ws_bytes;
   if (M < 0 || K < 0) return FM_ERR_SHAPE;
   if (M == 0) return FM_OK;
   if (!X && K > 0) return FM_ERR_NULL;
@@ -86,12 +87,11 @@ int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t l
   a.c_rs = a.c2_rs = ldy_row; a.c_cs = a.c2_cs = ldy_col;
   a.Ma = a.Nb = M; a.Kc = K;
   a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1;
-  return hip_status(launch_gemm_nt(a, static_cast<hipStream_t>(stream)));
+  return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, static_cast<hipStream_t>(stream)));
 }
 
 int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, float b, float c,
                       float* diag_out, void* ws, size_t ws_bytes, fm_stream_t stream) {
-  (void)ws; (void)ws_bytes;
   if (M < 0) return FM_ERR_SHAPE;
   if (M == 0) return FM_OK;
   if (!A || !P) return FM_ERR_NULL;
@@ -102,20 +102,19 @@ int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, f
                    overlaps(mat_range(diag_out, 1, M, M, 4), mat_range(P, M, M, ldp, 2))))
     return FM_ERR_ALIAS;
   GemmArgs a = {};
-  a.A = a.B = a.E = static_cast<const bf16_t*>(A); a.lda = a.ldb = a.lde = lda;
+  a.A = a.B = a.E = a.ET = static_cast<const bf16_t*>(A); a.lda = a.ldb = a.lde = a.ldet = lda;
   a.C = a.C2 = static_cast<bf16_t*>(P);
   a.c_rs = a.c2_rs = ldp; a.c_cs = a.c2_cs = 1;
   a.Ma = a.Nb = a.Kc = M;
   a.alpha = b; a.beta = c; a.symmetric = 1;
   a.diag_out = diag_out;
-  return hip_status(launch_gemm_nt(a, static_cast<hipStream_t>(stream)));
+  return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, static_cast<hipStream_t>(stream)));
 }
 
 int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt, const void* X,
                        int64_t ldx, void* Xout, int64_t ldo, void* XoutT, int64_t ldot, int M, int K,
                        float alpha, const float* row_alpha, void* ws, size_t ws_bytes,
                        fm_stream_t stream) {
-  (void)ws; (void)ws_bytes;
   if (M < 0 || K < 0) return FM_ERR_SHAPE;
   if (M == 0 || K == 0) return FM_OK;
   if (!P || !XT || !X) return FM_ERR_NULL;
@@ -137,12 +136,13 @@ int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt,
   a.A = static_cast<const bf16_t*>(P); a.lda = ldp;
   a.B = static_cast<const bf16_t*>(XT); a.ldb = ldxt;
   a.E = static_cast<const bf16_t*>(X); a.lde = ldx;
+  a.ET = a.B; a.ldet = ldxt;
   a.C = static_cast<bf16_t*>(Xout); a.c_rs = ldo; a.c_cs = 1;
   a.C2 = static_cast<bf16_t*>(XoutT); a.c2_rs = ldot; a.c2_cs = 1;
   a.Ma = M; a.Nb = K; a.Kc = M;
   a.alpha = alpha; a.beta = 1.0f; a.symmetric = 0;
   a.row_alpha = row_alpha;
-  return hip_status(launch_gemm_nt(a, static_cast<hipStream_t>(stream)));
+  return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, static_cast<hipStream_t>(stream)));
 }
 
 size_t fm_sumsq_workspace_bytes(void) { return kSumsqBlocks * sizeof(float); }

@@ -225,7 +225,7 @@ static int launch_cfg(GemmArgs a, bool aligned, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-int launch_gemm_nt(GemmArgs a, hipStream_t stream) {
+int launch_gemm_general(GemmArgs a, hipStream_t stream) {
   const bool aligned = (a.lda % 8 == 0) && (a.ldb % 8 == 0) && (a.Kc % 8 == 0) &&
                        ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0) &&
                        ((reinterpret_cast<uintptr_t>(a.B) & 15) == 0);
@@ -235,6 +235,12 @@ int launch_gemm_nt(GemmArgs a, hipStream_t stream) {
   const int64_t work_tiles = a.symmetric ? (big_tiles + (a.Ma + 255) / 256) / 2 : big_tiles;
   if (work_tiles >= 256) return launch_cfg<256, 256, 2, 4>(a, aligned, stream);
   return launch_cfg<128, 128, 2, 2>(a, aligned, stream);
+}
+
+int launch_gemm_nt(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
+  if (gemm_fast_eligible(a) && ws && ws_bytes >= gemm_fast_workspace_bytes(a.Ma, a.Nb, a.symmetric != 0))
+    return launch_gemm_fast(a, ws, ws_bytes, stream);
+  return launch_gemm_general(a, stream);
 }
 
 }  // namespace fm

@@ -1,0 +1,525 @@
+// Fast path of the bf16 NT contraction for gfx950: 256x256 output tiles, 4 waves (one per SIMD) of
+// 128x128 each, 64-wide k stages copied global -> LDS by the DMA form of global_load (no VGPR
+// staging), two LDS stages.
+//
+// Schedule.  One workgroup per CU.  Tiles are taken in rounds of `grid` whole tiles: all workgroups
+// start a tile together and walk k in step, so the workgroups of one XCD, which hold a compact
+// block of tiles, find each other's operand panels in their shared L2.  What is left after the
+// last full round (fewer tiles than workgroups) is cut along k into `split` parts per tile, one
+// part per workgroup, so that the last round is as short as its share of the work; the parts go to
+// memory as fp32 and a second, small kernel adds them in part order and runs the epilogue.
+#include "fm_internal.h"
+#include <cstdlib>
+
+namespace fm {
+
+namespace {
+
+constexpr int BM = 256, BN = 256, BKF = 64;
+constexpr int ROWB = BKF * 2;               // bytes per LDS row
+constexpr int OPER_BYTES = BM * ROWB;       // one operand stage: 32 KiB
+constexpr int PART_FLOATS = BM * BN;        // one fp32 partial tile
+
+#define FM_LDS_ADDR(p) ((uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(p)))
+
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+// One wave-wide global -> LDS copy of 16 bytes per lane: lane l lands at lds_base + 16*l.
+// The compiler does not see the LDS write, so every use is ordered by hand with
+// s_waitcnt vmcnt + s_barrier before the data is read.
+__device__ __forceinline__ void dma16(uint32_t voff, const void* sbase, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(sbase), "s"(lds_base) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+__device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
+  float fT = (float)(2 * T + 1);
+  int ii = (int)((fT - __builtin_sqrtf(fT * fT - 8.0f * (float)t)) * 0.5f);
+  if (ii < 0) ii = 0;
+  if (ii > T - 1) ii = T - 1;
+  while (ii > 0 && (ii * T - (ii * (ii - 1)) / 2) > t) --ii;
+  while (ii + 1 < T && ((ii + 1) * T - ((ii + 1) * ii) / 2) <= t) ++ii;
+  i = ii;
+  j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
+}
+
+#define FM_MFMA(i, j, FA, FB) \
+  acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[i], FB[j], acc[i][j], 0, 0, 0)
+
+struct Frag { bf16x8_t a[4], b[4]; };
+
+__device__ __forceinline__ void read_frags(Frag& f, const unsigned char* sa, const unsigned char* sb,
+                                           const uint32_t (&ao)[4], const uint32_t (&bo)[4], int ks) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.a[i] = *reinterpret_cast<const bf16x8_t*>(sa + (ao[i] ^ (ks << 5)));
+#pragma unroll
+  for (int j = 0; j < 4; ++j) f.b[j] = *reinterpret_cast<const bf16x8_t*>(sb + (bo[j] ^ (ks << 5)));
+}
+
+// 16 MFMAs of one k16 substep; the 8 fragment reads of the next substep ride on the first 8.
+__device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
+                                      const unsigned char* sa, const unsigned char* sb,
+                                      const uint32_t (&ao)[4], const uint32_t (&bo)[4], int ks_next) {
+  read_frags(nxt, sa, sb, ao, bo, ks_next);
+#pragma unroll
+  for (int q = 0; q < 16; ++q) FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// Last substep of a stage.  After the barrier every wave holds its last fragments of this stage in
+// registers and the other stage has landed, so the 16 MFMAs run interleaved with the DMA that
+// refills this stage (16 copies) and with the first fragment reads of the other stage.
+__device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
+                                           const unsigned char* nsa, const unsigned char* nsb,
+                                           const uint32_t (&ao)[4], const uint32_t (&bo)[4],
+                                           const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                           const bf16_t* gA, const bf16_t* gB, uint32_t ldsA, uint32_t ldsB) {
+  wait_vmcnt<0>();
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    if (q < 8) dma16(voA[q], gA, ldsA + q * 4096);
+    else dma16(voB[q - 8], gB, ldsB + (q - 8) * 4096);
+    if (q < 4) nxt.a[q] = *reinterpret_cast<const bf16x8_t*>(nsa + ao[q]);
+    else if (q < 8) nxt.b[q - 4] = *reinterpret_cast<const bf16x8_t*>(nsb + bo[q - 4]);
+    FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+__device__ __forceinline__ unsigned short f2bf(float v) {
+  return __builtin_bit_cast(unsigned short, (bf16_t)v);
+}
+__device__ __forceinline__ float bfbits2f(unsigned short h) {
+  return __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+
+
+// ---- staging of one half (64 rows x 128 columns) of a wave's accumulators in LDS -----------------
+constexpr int STG_PITCH = 68;                          // floats per column: 64 rows + 4 of padding
+constexpr int STG_WAVE_FLOATS = 128 * STG_PITCH;       // 34816 bytes per wave
+constexpr int SMEM_BYTES = 4 * STG_WAVE_FLOATS * 4;    // 139264 >= the 131072 of the operand stages
+
+// float index of row r (0..63) of column c (0..127): 4-row groups are XOR-swizzled with c/8
+__device__ __forceinline__ int stg_idx(int c, int r) { return c * STG_PITCH + (r ^ (((c >> 3) & 15) << 2)); }
+
+__device__ __forceinline__ void stage_store(const f32x16_t (&acc)[4][4], int h, float* stg, int lane) {
+  const int c = lane & 31, rg = 4 * (lane >> 5);
+#pragma unroll
+  for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = 2 * h + ii;
+        f32x4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        *reinterpret_cast<f32x4_t*>(stg + stg_idx(32 * j + c, 32 * ii + 8 * q + rg)) = v;
+      }
+}
+
+// the 128 x 64 floats of the staged half, in staging order, to a partial-tile slot (coalesced)
+__device__ __forceinline__ void copy_stage_to_ws(const float* stg, float* dst, int lane) {
+#pragma unroll 8
+  for (int it = 0; it < 32; ++it) {
+    const int idx = it * 64 + lane;             // 16-byte unit: column idx/16, 4-row group idx%16
+    const f32x4_t v = *reinterpret_cast<const f32x4_t*>(stg + (idx >> 4) * STG_PITCH + (idx & 15) * 4);
+    *reinterpret_cast<f32x4_t*>(dst + idx * 4) = v;
+  }
+}
+
+// sum of the `nparts` parts of one staged half, in part order, back into staging layout; this wave
+// takes the 16-byte units it_begin*64 .. it_end*64.  Loads go out eight parts at a time.
+__device__ __forceinline__ void sum_parts_to_stage(const float* parts, int nparts, float* stg, int lane,
+                                                   int it_begin, int it_end) {
+  for (int it = it_begin; it < it_end; ++it) {
+    const int idx = it * 64 + lane;
+    f32x4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int t0 = 0; t0 < nparts; t0 += 8) {
+      f32x4_t x[8];
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const int tt = (t0 + t < nparts) ? t0 + t : nparts - 1;   // clamped; the value is dropped below
+        x[t] = *reinterpret_cast<const f32x4_t*>(parts + (size_t)tt * PART_FLOATS + idx * 4);
+      }
+#pragma unroll
+      for (int t = 0; t < 8; ++t) if (t0 + t < nparts) v += x[t];
+    }
+    *reinterpret_cast<f32x4_t*>(stg + (idx >> 4) * STG_PITCH + (idx & 15) * 4) = v;
+  }
+}
+
+// value stored for accumulator a at (row, col): a itself, or al * e + beta * a; spelled with an
+// explicit multiply and fma so that the two passes below produce the same bits
+__device__ __forceinline__ float epi_value(float a, float e, float al, float beta, bool has_e) {
+  return has_e ? __builtin_fmaf(al, e, __fmul_rn(beta, a)) : a;
+}
+
+// Epilogue of the staged half h of the wave's block: rows m0 + wm*128 + 64h .. +64, columns
+// n0 + wn*128 .. +128.  Pass 1 writes C2 (the transposed copy) 8 rows x 1 column per lane, pass 2
+// writes C 1 row x 8 columns per lane; both 16 bytes per lane and coalesced.  HAS_E: the epilogue
+// operand is present; HAS_RA: so is the per-row addition to alpha; DIAG: this is a diagonal tile
+// of a symmetric product (masks, and the fp32 diagonal if it is asked for).
+template <bool HAS_E, bool HAS_RA, bool DIAG>
+__device__ __forceinline__ void epilogue_half_t(const GemmArgs& g, const float* stg, int ti, int tj,
+                                                int wm, int wn, int h, int lane, int it_begin, int it_end) {
+  const int row_base = ti * BM + wm * 128 + 64 * h;    // global row of staged row 0
+  const int col_base = tj * BN + wn * 128;             // global column of staged column 0
+  const float alpha = g.alpha, beta = g.beta;
+  const bool dout = DIAG && g.diag_out != nullptr;
+  if (g.C2) {
+    unsigned short* C2 = reinterpret_cast<unsigned short*>(g.C2);
+    const unsigned short* ET = reinterpret_cast<const unsigned short*>(g.ET);
+#pragma unroll 4
+    for (int it = it_begin; it < it_end; ++it) {
+      const int idx = it * 64 + lane;
+      const int c = idx >> 3, r0 = (idx & 7) * 8;      // column c, rows r0 .. r0+7 of the staged half
+      const int col = col_base + c, row = row_base + r0;
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0));
+      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0 + 4));
+      float a[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      union { uint4 v; unsigned short s[8]; } e, o;
+      float al[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) al[k] = alpha;
+      if (HAS_E) e.v = *reinterpret_cast<const uint4*>(ET + (int64_t)col * g.ldet + row);
+      if (HAS_RA) {
+        const f32x4_t r_lo = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row);
+        const f32x4_t r_hi = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { al[k] += r_lo[k]; al[k + 4] += r_hi[k]; }
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        float v = epi_value(a[k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al[k], beta, HAS_E);
+        if (dout && row + k == col) v = 0.0f;          // pass 2 hands the fp32 diagonal out
+        o.s[k] = f2bf(v);
+      }
+      unsigned short* dst = C2 + (int64_t)col * g.c2_rs + row;
+      // diagonal tile: mirror only what lies strictly above the diagonal (col > row + k); a group
+      // of 8 rows is all above it, all on or below it, or straddles it
+      if (!DIAG || col > row + 7) {
+        *reinterpret_cast<uint4*>(dst) = o.v;
+      } else if (col > row) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) if (col > row + k) dst[k] = o.s[k];
+      }
+    }
+  }
+  if (g.C) {
+    unsigned short* C = reinterpret_cast<unsigned short*>(g.C);
+    const unsigned short* E = reinterpret_cast<const unsigned short*>(g.E);
+#pragma unroll 4
+    for (int it = it_begin; it < it_end; ++it) {
+      const int idx = it * 64 + lane;
+      const int r = idx >> 4, c0 = (idx & 15) * 8;     // row r, columns c0 .. c0+7 of the staged half
+      const int row = row_base + r, col = col_base + c0;
+      float a[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) a[k] = stg[stg_idx(c0 + k, r)];
+      union { uint4 v; unsigned short s[8]; } e, o;
+      if (HAS_E) e.v = *reinterpret_cast<const uint4*>(E + (int64_t)row * g.lde + col);
+      float al = alpha;
+      if (HAS_RA) al += g.row_alpha[row];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        float v = epi_value(a[k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al, beta, HAS_E);
+        if (dout && row == col + k) { g.diag_out[row] = v; v = 0.0f; }
+        o.s[k] = f2bf(v);
+      }
+      unsigned short* dst = C + (int64_t)row * g.c_rs + col;
+      // diagonal tile: keep what lies on or above the diagonal (col + k >= row); the rest of the
+      // row comes from pass 1 of the mirrored position, i.e. from the same accumulator
+      if (!DIAG || col >= row) {
+        *reinterpret_cast<uint4*>(dst) = o.v;
+      } else if (col + 7 >= row) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) if (col + k >= row) dst[k] = o.s[k];
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ void epilogue_half(const GemmArgs& g, const float* stg, int ti, int tj,
+                                              int wm, int wn, int h, int lane, int it_begin = 0, int it_end = 16) {
+  const bool diag = g.symmetric && ti == tj;
+  if (!g.E) {
+    if (diag) epilogue_half_t<false, false, true>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+    else epilogue_half_t<false, false, false>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+  } else if (diag) {
+    epilogue_half_t<true, false, true>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+  } else if (g.row_alpha) {
+    epilogue_half_t<true, true, false>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+  } else {
+    epilogue_half_t<true, false, false>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+  }
+}
+
+struct FastArgs {
+  GemmArgs g;
+  float* partials;      // rem * split fp32 tiles: part q of tail tile t is slot t * split + q
+  int nk;               // k stages per tile
+  int grid;             // workgroups launched (a multiple of 8, or fewer than 8)
+  int rounds;           // full rounds: tiles [0, rounds * grid) are computed whole
+  int rem;              // tiles of the last, partial round
+  int split;            // k parts per tile of the last round (1: whole tiles, nothing to add up)
+  int dbg;              // tuning aid: bit 0 skips the epilogue, bit 1 skips the main loop
+};
+
+// Position in the schedule -> tile coordinates.  Tiles are visited in 8x8 blocks (row-major over
+// the blocks, row-major inside a block; blocks below the diagonal are skipped and blocks on it are
+// triangles when the product is symmetric), so the ~32 tiles an XCD works on at any one time touch
+// about 8 + 8 operand panels instead of one panel per tile, and its L2 serves most of the copies.
+__device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& ti, int& tj) {
+  constexpr int SB = 8;
+  const int nbm = (g.tiles_m + SB - 1) / SB, nbn = (g.tiles_n + SB - 1) / SB;
+  for (int I = 0; I < nbm; ++I) {
+    const int rows = (g.tiles_m - I * SB) < SB ? (g.tiles_m - I * SB) : SB;
+    for (int J = g.symmetric ? I : 0; J < nbn; ++J) {
+      const int cols = (g.tiles_n - J * SB) < SB ? (g.tiles_n - J * SB) : SB;
+      const bool tri = g.symmetric && I == J;
+      const int cnt = tri ? rows * (rows + 1) / 2 : rows * cols;
+      if (pos < cnt) {
+        int a, b;
+        if (tri) { tri_decode(pos, rows, a, b); } else { a = pos / cols; b = pos - a * cols; }
+        ti = I * SB + a;
+        tj = J * SB + b;
+        return;
+      }
+      pos -= cnt;
+    }
+  }
+  ti = tj = 0;   // not reached for pos < num_tiles
+}
+
+__global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
+  // two operand stages (A0 B0 A1 B1, 32 KiB each) during the main loop, the accumulator staging of
+  // the four waves afterwards
+  __shared__ __align__(1024) unsigned char smem[SMEM_BYTES];
+  unsigned char* const sA0 = smem;
+  unsigned char* const sB0 = smem + OPER_BYTES;
+  unsigned char* const sA1 = smem + 2 * OPER_BYTES;
+  unsigned char* const sB1 = smem + 3 * OPER_BYTES;
+
+  const GemmArgs& g = p.g;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous block of positions
+  // so that the tiles it holds at any one time are neighbours in the blocked tile order.
+  int w = (int)blockIdx.x;
+  if (p.grid >= 8) w = (w & 7) * (p.grid >> 3) + (w >> 3);
+
+  const uint32_t lA0 = FM_LDS_ADDR(sA0) + wave * 1024, lB0 = FM_LDS_ADDR(sB0) + wave * 1024;
+  const uint32_t lA1 = FM_LDS_ADDR(sA1) + wave * 1024, lB1 = FM_LDS_ADDR(sB1) + wave * 1024;
+
+  // per-lane fragment offsets inside an operand stage (row = lane % 32, k half = lane / 32)
+  uint32_t ao[4], bo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ra = wm * 128 + i * 32 + (lane & 31);
+    ao[i] = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
+    const int rb = wn * 128 + i * 32 + (lane & 31);
+    bo[i] = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
+  }
+
+  for (int round = 0; round <= p.rounds; ++round) {
+    int pos, kb, ke, part = 0;
+    if (round < p.rounds) {
+      pos = round * p.grid + w; kb = 0; ke = p.nk;
+    } else {
+      if (w >= p.rem * p.split) break;
+      pos = p.rounds * p.grid + w / p.split;
+      part = w - (w / p.split) * p.split;
+      kb = (int)((long long)p.nk * part / p.split);
+      ke = (int)((long long)p.nk * (part + 1) / p.split);
+    }
+    const int n = ke - kb;
+
+    int ti, tj;
+    tile_at(g, pos, ti, tj);
+    const int m0 = ti * BM, n0 = tj * BN;
+
+    // DMA copy q of this wave fills LDS rows (q*4 + wave)*8 .. +8 of an operand stage (the output
+    // is a whole number of tiles on this path, so every row exists)
+    uint32_t voA[8], voB[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int row = (q * 4 + wave) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ swz(row);
+      voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
+      voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
+    }
+    const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
+    const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
+
+    f32x16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // ---- main loop over k stages kb .. ke-1 ----------------------------------------------------
+    {
+      Frag f0, f1;
+      const int k1 = n > 1 ? 1 : 0;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) { dma16(voA[q], gA, lA0 + q * 4096); dma16(voB[q], gB, lB0 + q * 4096); }
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        dma16(voA[q], gA + k1 * BKF, lA1 + q * 4096);
+        dma16(voB[q], gB + k1 * BKF, lB1 + q * 4096);
+      }
+      wait_vmcnt<16>();
+      __syncthreads();
+      read_frags(f0, sA0, sB0, ao, bo, 0);
+      // stages go through the loop in pairs (a loop with a second exit in the middle makes the
+      // register allocator give up on keeping the accumulators in place); an odd last stage follows
+      int it = 0;
+      if (p.dbg & 2) it = n & ~1;
+      for (; it + 2 <= n; it += 2) {
+        phase(acc, f0, f1, sA0, sB0, ao, bo, 1);
+        phase(acc, f1, f0, sA0, sB0, ao, bo, 2);
+        phase(acc, f0, f1, sA0, sB0, ao, bo, 3);
+        {
+          const int kn = (it + 2 < n) ? it + 2 : n - 1;
+          tail_phase(acc, f1, f0, sA1, sB1, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA0, lB0);
+        }
+        phase(acc, f0, f1, sA1, sB1, ao, bo, 1);
+        phase(acc, f1, f0, sA1, sB1, ao, bo, 2);
+        phase(acc, f0, f1, sA1, sB1, ao, bo, 3);
+        {
+          const int kn = (it + 3 < n) ? it + 3 : n - 1;
+          tail_phase(acc, f1, f0, sA0, sB0, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA1, lB1);
+        }
+      }
+      if (it < n) {   // one stage left: it sits in stage 0 and its first fragments are in f0
+        phase(acc, f0, f1, sA0, sB0, ao, bo, 1);
+        phase(acc, f1, f0, sA0, sB0, ao, bo, 2);
+        phase(acc, f0, f1, sA0, sB0, ao, bo, 3);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) FM_MFMA(q >> 2, q & 3, f1.a, f1.b);
+      }
+      wait_vmcnt<0>();
+      __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
+    }
+
+    // ---- accumulators -> LDS, then everything else from LDS with plain loops --------------------
+    // Register 4q+e of lane l in MFMA tile (i, j) is row 32i + 8q + 4(l/32) + e, column 32j + l%32
+    // of the wave's 128x128 block: four consecutive rows of one column.  Each wave parks one half of
+    // its block (64 rows x 128 columns, fp32) at a time in its own LDS region, column-major
+    // (T[c][r], 4-row groups XOR-swizzled by c/8), which both passes below read without conflicts.
+    const bool split = (n != p.nk);
+    float* const stg = reinterpret_cast<float*>(smem) + wave * STG_WAVE_FLOATS;
+    float* const slot = p.partials + (size_t)((pos - p.rounds * p.grid) * p.split + part) * PART_FLOATS;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      stage_store(acc, h, stg, lane);
+      if (split) copy_stage_to_ws(stg, slot + (wave * 2 + h) * (128 * 64), lane);
+      else if (!(p.dbg & 1)) epilogue_half(g, stg, ti, tj, wm, wn, h, lane);
+    }
+    __syncthreads();   // the next tile's copies land in the memory the staging just used
+  }
+}
+
+// Second kernel of a split last round: one workgroup per (tail tile, 128x128 block, half).  Its four
+// waves add the parts in part order, so the bits do not depend on which workgroup finished when,
+// into one staging buffer, and then share the iterations of the same epilogue the main kernel runs.
+__global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
+  __shared__ __align__(16) float stg[STG_WAVE_FLOATS];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int t = blockIdx.x >> 3, blk = (blockIdx.x >> 1) & 3, h = blockIdx.x & 1;
+  int ti, tj;
+  tile_at(p.g, p.rounds * p.grid + t, ti, tj);
+  sum_parts_to_stage(p.partials + (size_t)t * p.split * PART_FLOATS + (blk * 2 + h) * (128 * 64), p.split, stg,
+                     lane, wave * 8, wave * 8 + 8);
+  __syncthreads();
+  epilogue_half(p.g, stg, ti, tj, blk >> 1, blk & 1, h, lane, wave * 4, wave * 4 + 4);
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+// grid, rounds, remainder and split of the schedule for `num_tiles` tiles of `nk` k stages
+static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
+  int grid = 256;                                   // one workgroup per CU (136 KiB of LDS each)
+  if (const char* e = std::getenv("FLASHMUON_GRID")) grid = std::atoi(e);   // tuning aid
+  if (grid > num_tiles) grid = num_tiles;           // rem * split never exceeds the grid below
+  if (grid >= 8) grid &= ~7;
+  if (grid < 1) grid = 1;
+  f.grid = grid;
+  f.rounds = num_tiles / grid;
+  f.rem = num_tiles % grid;
+  f.split = 1;
+  if (f.rem > 0) {
+    int s = grid / f.rem;                           // parts that fit in one round of workgroups
+    if (s > nk) s = nk;
+    if (s > 32) s = 32;                             // bounds the partial-tile traffic
+    f.split = s < 1 ? 1 : s;
+  }
+}
+
+bool gemm_fast_eligible(const GemmArgs& a) {
+  if (a.Kc < BKF || a.Kc % BKF != 0) return false;
+  if (a.lda % 8 != 0 || a.ldb % 8 != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(a.A) & 15) || (reinterpret_cast<uintptr_t>(a.B) & 15)) return false;
+  if (a.Ma % BM != 0 || a.Nb % BN != 0) return false;           // whole tiles only: no edge masks here
+  // in-tile byte offsets stay below 2^31
+  if (a.lda >= (1 << 21) || a.ldb >= (1 << 21)) return false;
+  if (a.C && a.c_cs != 1) return false;
+  if (a.C2 && a.c2_cs != 1) return false;
+  // 16-byte accesses of the epilogue
+  if (a.C && (a.c_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C) & 15))) return false;
+  if (a.C2 && (a.c2_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C2) & 15))) return false;
+  if (a.E && a.C && (a.lde % 8 != 0 || (reinterpret_cast<uintptr_t>(a.E) & 15))) return false;
+  if (a.E && a.C2 && (!a.ET || a.ldet % 8 != 0 || (reinterpret_cast<uintptr_t>(a.ET) & 15))) return false;
+  if (a.row_alpha && (reinterpret_cast<uintptr_t>(a.row_alpha) & 15)) return false;
+  // small problems: 128x128 tiles fill the chip better than few 256x256 tiles
+  // (FLASHMUON_FAST_MIN_UNITS overrides the threshold, e.g. 0 to exercise this path on small inputs)
+  const long long tm = a.Ma / BM, tn = a.Nb / BN;
+  const long long tiles = a.symmetric ? tm * (tm + 1) / 2 : tm * tn;
+  static const long long min_units = [] {
+    const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS");
+    return e ? std::atoll(e) : 8192LL;
+  }();
+  if (tiles * (a.Kc / BKF) < min_units) return false;
+  return true;
+}
+
+size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric) {
+  (void)Ma; (void)Nb; (void)symmetric;
+  return (size_t)256 * PART_FLOATS * sizeof(float);   // rem * split <= grid <= 256 partial tiles
+}
+
+int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
+  a.tiles_m = a.Ma / BM;
+  a.tiles_n = a.Nb / BN;
+  a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;
+  FastArgs f;
+  f.g = a;
+  f.nk = a.Kc / BKF;
+  fast_schedule(a.num_tiles, f.nk, f);
+  f.dbg = 0;
+  if (const char* e = std::getenv("FLASHMUON_DBG")) f.dbg = std::atoi(e);
+  f.partials = static_cast<float*>(ws);
+  if (f.split > 1 && (!ws || ws_bytes < (size_t)f.rem * f.split * PART_FLOATS * sizeof(float))) return -1;
+  hipLaunchKernelGGL(gemm_nt_rounds_kernel, dim3(f.grid), dim3(256), 0, stream, f);
+  if (f.split > 1)
+    hipLaunchKernelGGL(gemm_nt_reduce_kernel, dim3(f.rem * 8), dim3(256), 0, stream, f);
+  return (int)hipGetLastError();
+}
+
+}  // namespace fm

@@ -22,6 +22,7 @@ struct GemmArgs {
   const bf16_t* A;  int64_t lda;
   const bf16_t* B;  int64_t ldb;
   const bf16_t* E;  int64_t lde;
+  const bf16_t* ET; int64_t ldet;   // optional: the same operand transposed, ET[j][i] == E[i][j]
   bf16_t* C;  int64_t c_rs, c_cs;
   bf16_t* C2; int64_t c2_rs, c2_cs;
   int Ma, Nb, Kc;
@@ -33,8 +34,14 @@ struct GemmArgs {
   int num_tiles;          // tiles actually computed (triangular count when symmetric)
 };
 
-// Enqueue the contraction described by `args` on `stream`.  Returns a hipError_t value.
-int launch_gemm_nt(GemmArgs args, hipStream_t stream);
+// Enqueue the contraction described by `args` on `stream`, on the 256x256 stream-K path when the
+// shape, the alignment and the workspace allow it and on the general tiled path otherwise.
+// Returns a hipError_t value.
+int launch_gemm_nt(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
+int launch_gemm_general(GemmArgs args, hipStream_t stream);
+bool gemm_fast_eligible(const GemmArgs& a);
+size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric);
+int launch_gemm_fast(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
 
 int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
                  float* partials, hipStream_t stream);

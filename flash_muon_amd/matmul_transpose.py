@@ -36,7 +36,7 @@ def matmul_transpose_assign(d_in, d_out):
     ldx = d_in.stride(0) if K > 0 and M > 1 else max(K, 1)
     lib = _lib.load()
     with torch.cuda.device(d_in.device):
-        ws, ws_bytes = _lib.workspace(lib.fm_syrk_workspace_bytes(M, K), d_in.device)
+        ws, ws_bytes = _lib.workspace(lib.fm_gemm_workspace_bytes(M, M), d_in.device)
         st = lib.fm_syrk_bf16(d_in.data_ptr(), ldx, d_out.data_ptr(),
                               d_out.stride(0) if M > 1 else M, d_out.stride(1) if M > 1 else 1,
                               M, K, ws.data_ptr() if ws is not None else None, ws_bytes,

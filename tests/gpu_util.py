@@ -17,7 +17,7 @@ def syrk(lib, X, Y=None):
     M, K = X.shape
     if Y is None:
         Y = torch.empty(M, M, dtype=torch.bfloat16, device=X.device)
-    ws = _ws(lib.fm_syrk_workspace_bytes(M, K), X.device)
+    ws = _ws(lib.fm_gemm_workspace_bytes(M, M), X.device)
     st = lib.fm_syrk_bf16(X.data_ptr(), X.stride(0), Y.data_ptr(), Y.stride(0), Y.stride(1), M, K,
                           ws.data_ptr(), ws.numel(), _stream(X))
     _lib.check("fm_syrk_bf16", st)
@@ -29,7 +29,7 @@ def syrk_poly(lib, A, b, c, split_diag=False):
     M = A.size(0)
     P = torch.empty(M, M, dtype=torch.bfloat16, device=A.device)
     d = torch.empty(M, dtype=torch.float32, device=A.device) if split_diag else None
-    ws = _ws(lib.fm_syrk_workspace_bytes(M, M), A.device)
+    ws = _ws(lib.fm_gemm_workspace_bytes(M, M), A.device)
     st = lib.fm_syrk_poly_bf16(A.data_ptr(), A.stride(0), P.data_ptr(), P.stride(0), M, b, c,
                                d.data_ptr() if split_diag else None,
                                ws.data_ptr(), ws.numel(), _stream(A))
@@ -43,7 +43,7 @@ def gemm_axpby(lib, P, X, a, want_x=True, want_xt=True, XT=None, row_alpha=None)
         XT = X.T.contiguous()
     Xo = torch.empty(M, K, dtype=torch.bfloat16, device=X.device) if want_x else None
     XoT = torch.empty(K, M, dtype=torch.bfloat16, device=X.device) if want_xt else None
-    ws = _ws(lib.fm_syrk_workspace_bytes(M, max(M, K)), X.device)
+    ws = _ws(lib.fm_gemm_workspace_bytes(M, K), X.device)
     st = lib.fm_gemm_axpby_bf16(P.data_ptr(), P.stride(0), XT.data_ptr(), XT.stride(0),
                                 X.data_ptr(), X.stride(0),
                                 Xo.data_ptr() if want_x else None, Xo.stride(0) if want_x else 0,

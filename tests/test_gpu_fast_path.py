@@ -1,0 +1,88 @@
+"""The 256x256 stream-K path of the GEMM-shaped kernels.  It is chosen by shape (whole 256-tiles, k a
+multiple of 64, enough k stages to share out); FLASHMUON_FAST_MIN_UNITS=0 is set here, before the
+library is loaded, so that small inputs take it too and the split-tile hand-over is exercised with
+few, many and uneven parts per tile.  Integer-valued inputs make every comparison bit-exact."""
+import os
+
+os.environ["FLASHMUON_FAST_MIN_UNITS"] = "0"
+
+import pytest
+import torch
+
+from flash_muon_amd import matmul_transpose
+from tests import gpu_util
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _ints(shape, seed, lo=-2, hi=2):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi + 1, shape, generator=g).float().bfloat16()
+
+
+def _exact(x):   # exact integer matrix product in fp64, then the single bf16 rounding
+    return x.float().bfloat16()
+
+
+# (M, K): 1 tile and 1 stage; odd stage counts; many tiles; one tile split over many workgroups
+SYRK_SHAPES = [(256, 64), (256, 192), (256, 4096), (512, 320), (768, 1024), (1024, 576), (2048, 2048), (1280, 8192)]
+
+
+@pytest.mark.parametrize("M,K", SYRK_SHAPES)
+def test_syrk_fast_integer_bit_exact(lib, M, K):
+    X = _ints((M, K), M + K)
+    want = _exact(X.double() @ X.double().T)
+    Y = gpu_util.syrk(lib, X.to(DEV))
+    assert torch.equal(Y.cpu(), want)
+    assert torch.equal(Y, Y.T)
+    # a second run into a poisoned output gives the same bits (no dependence on arrival order)
+    Y2 = torch.full_like(Y, 7.0)
+    gpu_util.syrk(lib, X.to(DEV), Y2)
+    assert torch.equal(Y2, Y)
+
+
+@pytest.mark.parametrize("M", [256, 512, 1024, 1536])
+def test_poly_fast_integer_bit_exact(lib, M):
+    g = torch.Generator().manual_seed(M)
+    A = torch.randint(-1, 2, (M, M), generator=g)
+    A = (torch.triu(A) + torch.triu(A, 1).T).float().bfloat16()
+    Ad = A.double()
+    full = Ad + 2 * (Ad @ Ad)
+    assert torch.equal(gpu_util.syrk_poly(lib, A.to(DEV), 1.0, 2.0).cpu(), _exact(full))
+    P, d = gpu_util.syrk_poly(lib, A.to(DEV), 1.0, 2.0, split_diag=True)
+    assert torch.equal(d.cpu().double(), torch.diagonal(full))
+    assert torch.equal(P.cpu(), _exact(full - torch.diag(torch.diagonal(full))))
+    assert torch.equal(P, P.T)
+
+
+@pytest.mark.parametrize("M,K", [(256, 256), (256, 1280), (512, 768), (1024, 2048), (768, 4096)])
+def test_axpby_fast_integer_bit_exact(lib, M, K):
+    P = _ints((M, M), 3 * M + K, -1, 1)
+    X = _ints((M, K), 5 * M + K)
+    d = torch.arange(M, dtype=torch.float32) % 3 - 1            # per-row addition to a
+    want = _exact((2 + d.double())[:, None] * X.double() + P.double() @ X.double())
+    Xo, XoT = gpu_util.gemm_axpby(lib, P.to(DEV), X.to(DEV), 2.0, row_alpha=d.to(DEV))
+    assert torch.equal(Xo.cpu(), want)
+    assert torch.equal(XoT.cpu(), want.T)
+    only_t = gpu_util.gemm_axpby(lib, P.to(DEV), X.to(DEV), 2.0, want_x=False, row_alpha=d.to(DEV))[1]
+    assert torch.equal(only_t.cpu(), want.T)
+    only_x = gpu_util.gemm_axpby(lib, P.to(DEV), X.to(DEV), 2.0, want_xt=False, row_alpha=d.to(DEV))[0]
+    assert torch.equal(only_x.cpu(), want)
+
+
+def test_fast_and_general_paths_agree_on_gaussian_input(lib):
+    """Same input through the stream-K path (with workspace) and the tiled path (without): both are
+    one bf16 rounding of an fp32 sum, so they agree to within that rounding."""
+    g = torch.Generator().manual_seed(5)
+    X = torch.randn(1024, 2048, generator=g).bfloat16().to(DEV)
+    fast = gpu_util.syrk(lib, X)
+    slow = torch.empty_like(fast)
+    st = lib.fm_syrk_bf16(X.data_ptr(), X.stride(0), slow.data_ptr(), slow.stride(0), 1, 1024, 2048, None, 0,
+                          gpu_util._stream(X))
+    assert st == 0
+    assert torch.equal(fast, fast.T) and torch.equal(slow, slow.T)
+    ref = X.float() @ X.float().T
+    for Y in (fast, slow):
+        assert float((Y.float() - ref).norm() / ref.norm()) < 3e-3
+    assert torch.equal(matmul_transpose(X), fast)
