@@ -23,6 +23,12 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 DIM = 8192
+# L2-miss traffic of one 8192^2 call (main kernel + the kernel that adds up the split last round),
+# from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
+# 128 MiB device copy (FETCH_SIZE reads half of the copied bytes there, WRITE_SIZE all of them):
+# (559.7e3 + 32.9e3) KiB * 2.0 fetched + (203.6e3 + 3.5e3) KiB written.  The commands and the raw
+# readings are in profiles/syrk_bf16_8192_traffic.md.
+TRAFFIC_BYTES = int((559.7e3 + 32.9e3) * 1024 * 2.0 + (203.6e3 + 3.5e3) * 1024 * 1.0)
 
 
 def _time_gpu(fn, steps, warmup, torch):
@@ -103,6 +109,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--no-extras", action="store_true", help="skip vendor GEMM, Newton-Schulz and Muon.step timings")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 128 MiB device-to-device copy, the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path is built and measured on a single MI355X "
@@ -123,6 +132,10 @@ def main():
     torch.cuda.empty_cache()
     ms = _time_gpu(lambda: matmul_transpose_assign(Xd, Y), args.steps, args.warmup, torch)
     assert torch.equal(Y, Y.T), "output is not symmetric"
+    if args.copy_calibration:
+        Z = torch.empty_like(Xd)
+        Z.copy_(Xd)
+        torch.cuda.synchronize()
 
     useful = synthetic.syrk_useful_flop(DIM, DIM)
     tflops = useful / ms / 1e9
@@ -135,7 +148,8 @@ def main():
                    "M": DIM, "K": DIM},
         "effective_tflops": 2.0 * DIM * DIM * DIM / ms / 1e9,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": None},
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES,
+                     "flop_per_launch": useful, "kernel": "gemm_nt_rounds_kernel (+ gemm_nt_reduce_kernel)"},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = _cpu_baseline(X, torch)

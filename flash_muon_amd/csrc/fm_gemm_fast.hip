@@ -175,74 +175,95 @@ __device__ __forceinline__ void epilogue_half_t(const GemmArgs& g, const float* 
   const int col_base = tj * BN + wn * 128;             // global column of staged column 0
   const float alpha = g.alpha, beta = g.beta;
   const bool dout = DIAG && g.diag_out != nullptr;
+  // Iterations go four at a time, all loads of the four first: a load issued after a store has to
+  // wait for that store as well (one counter tracks both), which would serialise the loop on the
+  // write latency.
   if (g.C2) {
     unsigned short* C2 = reinterpret_cast<unsigned short*>(g.C2);
     const unsigned short* ET = reinterpret_cast<const unsigned short*>(g.ET);
-#pragma unroll 4
-    for (int it = it_begin; it < it_end; ++it) {
-      const int idx = it * 64 + lane;
-      const int c = idx >> 3, r0 = (idx & 7) * 8;      // column c, rows r0 .. r0+7 of the staged half
-      const int col = col_base + c, row = row_base + r0;
-      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0));
-      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0 + 4));
-      float a[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      union { uint4 v; unsigned short s[8]; } e, o;
-      float al[8];
+    for (int it0 = it_begin; it0 < it_end; it0 += 4) {
+      f32x4_t lo[4], hi[4], r_lo[4], r_hi[4];
+      uint4 ev[4];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) al[k] = alpha;
-      if (HAS_E) e.v = *reinterpret_cast<const uint4*>(ET + (int64_t)col * g.ldet + row);
-      if (HAS_RA) {
-        const f32x4_t r_lo = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row);
-        const f32x4_t r_hi = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row + 4);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) { al[k] += r_lo[k]; al[k + 4] += r_hi[k]; }
+      for (int u = 0; u < 4; ++u) {
+        const int idx = (it0 + u) * 64 + lane;
+        const int c = idx >> 3, r0 = (idx & 7) * 8;    // column c, rows r0 .. r0+7 of the staged half
+        const int col = col_base + c, row = row_base + r0;
+        lo[u] = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0));
+        hi[u] = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0 + 4));
+        if (HAS_E) ev[u] = *reinterpret_cast<const uint4*>(ET + (int64_t)col * g.ldet + row);
+        if (HAS_RA) {
+          r_lo[u] = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row);
+          r_hi[u] = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row + 4);
+        }
       }
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        float v = epi_value(a[k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al[k], beta, HAS_E);
-        if (dout && row + k == col) v = 0.0f;          // pass 2 hands the fp32 diagonal out
-        o.s[k] = f2bf(v);
-      }
-      unsigned short* dst = C2 + (int64_t)col * g.c2_rs + row;
-      // diagonal tile: mirror only what lies strictly above the diagonal (col > row + k); a group
-      // of 8 rows is all above it, all on or below it, or straddles it
-      if (!DIAG || col > row + 7) {
-        *reinterpret_cast<uint4*>(dst) = o.v;
-      } else if (col > row) {
+      for (int u = 0; u < 4; ++u) {
+        const int idx = (it0 + u) * 64 + lane;
+        const int c = idx >> 3, r0 = (idx & 7) * 8;
+        const int col = col_base + c, row = row_base + r0;
+        const float a[8] = {lo[u][0], lo[u][1], lo[u][2], lo[u][3], hi[u][0], hi[u][1], hi[u][2], hi[u][3]};
+        union { uint4 v; unsigned short s[8]; } e, o;
+        if (HAS_E) e.v = ev[u];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) if (col > row + k) dst[k] = o.s[k];
+        for (int k = 0; k < 8; ++k) {
+          float al = alpha;
+          if (HAS_RA) al += (k < 4) ? r_lo[u][k & 3] : r_hi[u][k & 3];
+          float v = epi_value(a[k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al, beta, HAS_E);
+          if (dout && row + k == col) v = 0.0f;        // pass 2 hands the fp32 diagonal out
+          o.s[k] = f2bf(v);
+        }
+        unsigned short* dst = C2 + (int64_t)col * g.c2_rs + row;
+        // diagonal tile: mirror only what lies strictly above the diagonal (col > row + k); a group
+        // of 8 rows is all above it, all on or below it, or straddles it
+        if (!DIAG || col > row + 7) {
+          *reinterpret_cast<uint4*>(dst) = o.v;
+        } else if (col > row) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) if (col > row + k) dst[k] = o.s[k];
+        }
       }
     }
   }
   if (g.C) {
     unsigned short* C = reinterpret_cast<unsigned short*>(g.C);
     const unsigned short* E = reinterpret_cast<const unsigned short*>(g.E);
-#pragma unroll 4
-    for (int it = it_begin; it < it_end; ++it) {
-      const int idx = it * 64 + lane;
-      const int r = idx >> 4, c0 = (idx & 15) * 8;     // row r, columns c0 .. c0+7 of the staged half
-      const int row = row_base + r, col = col_base + c0;
-      float a[8];
+    for (int it0 = it_begin; it0 < it_end; it0 += 4) {
+      float a[4][8], ra[4];
+      uint4 ev[4];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) a[k] = stg[stg_idx(c0 + k, r)];
-      union { uint4 v; unsigned short s[8]; } e, o;
-      if (HAS_E) e.v = *reinterpret_cast<const uint4*>(E + (int64_t)row * g.lde + col);
-      float al = alpha;
-      if (HAS_RA) al += g.row_alpha[row];
+      for (int u = 0; u < 4; ++u) {
+        const int idx = (it0 + u) * 64 + lane;
+        const int r = idx >> 4, c0 = (idx & 15) * 8;   // row r, columns c0 .. c0+7 of the staged half
+        const int row = row_base + r, col = col_base + c0;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        float v = epi_value(a[k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al, beta, HAS_E);
-        if (dout && row == col + k) { g.diag_out[row] = v; v = 0.0f; }
-        o.s[k] = f2bf(v);
+        for (int k = 0; k < 8; ++k) a[u][k] = stg[stg_idx(c0 + k, r)];
+        if (HAS_E) ev[u] = *reinterpret_cast<const uint4*>(E + (int64_t)row * g.lde + col);
+        if (HAS_RA) ra[u] = g.row_alpha[row];
       }
-      unsigned short* dst = C + (int64_t)row * g.c_rs + col;
-      // diagonal tile: keep what lies on or above the diagonal (col + k >= row); the rest of the
-      // row comes from pass 1 of the mirrored position, i.e. from the same accumulator
-      if (!DIAG || col >= row) {
-        *reinterpret_cast<uint4*>(dst) = o.v;
-      } else if (col + 7 >= row) {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) if (col + k >= row) dst[k] = o.s[k];
+      for (int u = 0; u < 4; ++u) {
+        const int idx = (it0 + u) * 64 + lane;
+        const int r = idx >> 4, c0 = (idx & 15) * 8;
+        const int row = row_base + r, col = col_base + c0;
+        union { uint4 v; unsigned short s[8]; } e, o;
+        if (HAS_E) e.v = ev[u];
+        const float al = HAS_RA ? alpha + ra[u] : alpha;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          float v = epi_value(a[u][k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al, beta, HAS_E);
+          if (dout && row == col + k) { g.diag_out[row] = v; v = 0.0f; }
+          o.s[k] = f2bf(v);
+        }
+        unsigned short* dst = C + (int64_t)row * g.c_rs + col;
+        // diagonal tile: keep what lies on or above the diagonal (col + k >= row); the rest of the
+        // row comes from pass 1 of the mirrored position, i.e. from the same accumulator
+        if (!DIAG || col >= row) {
+          *reinterpret_cast<uint4*>(dst) = o.v;
+        } else if (col + 7 >= row) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) if (col + k >= row) dst[k] = o.s[k];
+        }
       }
     }
   }
