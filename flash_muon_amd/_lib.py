@@ -35,6 +35,9 @@ SIGNATURES = {
     "fm_newtonschulz_workspace_bytes": (_sz, [_i32, _i32]),
     "fm_newtonschulz_bf16": (_i32, [_vp, _i32, _i32, _i32, _i64, _vp, _i64, _i32, _f32, _f32, _f32,
                                     _f32, _vp, _sz, _vp]),
+    "fm_newtonschulz_batched_workspace_bytes": (_sz, [_i32, _i32, _i32]),
+    "fm_newtonschulz_batched_bf16": (_i32, [_vp, _i32, _i32, _i32, _i32, _i64, _vp, _i64, _i32, _f32, _f32,
+                                            _f32, _f32, _vp, _sz, _vp]),
     "fm_momentum_nesterov": (_i32, [_vp, _vp, _i32, _i64, _f32, _f32, _i32, _vp]),
     "fm_weight_update": (_i32, [_vp, _i32, _vp, _i64, _f32, _f32, _vp]),
 }

@@ -25,21 +25,25 @@ inline int hip_status(int hip_err) { return hip_err == 0 ? FM_OK : FM_ERR_LAUNCH
 // a workspace is only used when it is 256-byte aligned; otherwise the call runs without one
 inline void* usable_ws(void* ws) { return (reinterpret_cast<uintptr_t>(ws) % 256 == 0) ? ws : nullptr; }
 
-// workspace of fm_newtonschulz_bf16, carved in this order
+// workspace of fm_newtonschulz_batched_bf16, carved in this order; per-matrix arrays are
+// batch-major with the strides below
 struct NsLayout {
   size_t sumsq, partials, pdiag, x[2], xt[2], a, p, gemm, total;
+  size_t pdiag_stride;   // floats between the fp32 diagonals of consecutive matrices
 };
-NsLayout ns_layout(int rows, int cols) {
+NsLayout ns_layout(int batch, int rows, int cols) {
   const size_t M = (size_t)(rows < cols ? rows : cols), K = (size_t)(rows < cols ? cols : rows);
+  const size_t B = (size_t)batch;
   NsLayout l;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
-  l.sumsq = take(sizeof(float));
-  l.partials = take(kSumsqBlocks * sizeof(float));
-  l.pdiag = take(M * sizeof(float));
-  for (int i = 0; i < 2; ++i) { l.x[i] = take(M * K * 2); l.xt[i] = take(M * K * 2); }
-  l.a = take(M * M * 2);
-  l.p = take(M * M * 2);
+  l.sumsq = take(B * 64 * sizeof(float));                 // one float per matrix, 256 bytes apart
+  l.partials = take(B * kSumsqBlocks * sizeof(float));
+  l.pdiag_stride = align_up(M, 64);
+  l.pdiag = take(B * l.pdiag_stride * sizeof(float));
+  for (int i = 0; i < 2; ++i) { l.x[i] = take(B * M * K * 2); l.xt[i] = take(B * M * K * 2); }
+  l.a = take(B * M * M * 2);
+  l.p = take(B * M * M * 2);
   l.gemm = take(fm_gemm_workspace_bytes((int)M, (int)K));
   l.total = off;
   return l;
@@ -178,67 +182,114 @@ int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int64_t ldg
                                       static_cast<hipStream_t>(stream)));
 }
 
+size_t fm_newtonschulz_batched_workspace_bytes(int batch, int rows, int cols) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
+  return ns_layout(batch, rows, cols).total;
+}
+
 size_t fm_newtonschulz_workspace_bytes(int rows, int cols) {
-  if (rows <= 0 || cols <= 0) return 0;
-  return ns_layout(rows, cols).total;
+  return fm_newtonschulz_batched_workspace_bytes(1, rows, cols);
+}
+
+int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int rows, int cols,
+                                 int64_t ldg, void* const* out, int64_t ldout, int steps, float a,
+                                 float b, float c, float eps, void* ws, size_t ws_bytes,
+                                 fm_stream_t stream) {
+  if (bad_dtype(dtype)) return FM_ERR_DTYPE;
+  if (rows < 0 || cols < 0 || steps < 0 || batch < 0 || batch > kMaxBatch) return FM_ERR_SHAPE;
+  if (rows == 0 || cols == 0 || batch == 0) return FM_OK;
+  if (!G || !out) return FM_ERR_NULL;
+  if (ldg < cols || ldout < cols) return FM_ERR_STRIDE;
+  for (int i = 0; i < batch; ++i) {
+    if (!G[i] || !out[i]) return FM_ERR_NULL;
+    if (misaligned(G[i], dtype_size(dtype)) || misaligned(out[i], 2)) return FM_ERR_ALIGN;
+    const Range oi = mat_range(out[i], rows, cols, ldout, 2);
+    for (int j = 0; j < batch; ++j) {
+      if (overlaps(mat_range(G[j], rows, cols, ldg, dtype_size(dtype)), oi)) return FM_ERR_ALIAS;
+      if (j != i && overlaps(mat_range(out[j], rows, cols, ldout, 2), oi)) return FM_ERR_ALIAS;
+    }
+  }
+  const NsLayout l = ns_layout(batch, rows, cols);
+  if (!ws || ws_bytes < l.total) return FM_ERR_WORKSPACE;
+  if (reinterpret_cast<uintptr_t>(ws) % 256 != 0) return FM_ERR_ALIGN;
+
+  unsigned char* w = static_cast<unsigned char*>(ws);
+  void* gws = w + l.gemm;
+  const size_t gws_bytes = l.total - l.gemm;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  const bool tall = rows > cols;
+  const int M = tall ? cols : rows, K = tall ? rows : cols;
+  const int64_t mk = (int64_t)M * K, mm = (int64_t)M * M;
+
+  // The iteration runs on X (M x K) with M <= K.  G is X when it is wide and X^T when it is
+  // tall, so the scaled cast of G is X in one case and X^T in the other.
+  bf16_t* X = reinterpret_cast<bf16_t*>(w + l.x[0]);
+  bf16_t* XT = reinterpret_cast<bf16_t*>(w + l.xt[0]);
+  for (int i = 0; i < batch; ++i) {
+    float* sumsq = reinterpret_cast<float*>(w + l.sumsq) + 64 * i;
+    void* partials = w + l.partials + (size_t)i * kSumsqBlocks * sizeof(float);
+    int st = fm_sumsq(G[i], dtype, rows, cols, ldg, sumsq, partials, fm_sumsq_workspace_bytes(), stream);
+    if (st) return st;
+    if (steps == 0) st = fm_scale_cast_bf16(G[i], dtype, rows, cols, ldg, sumsq, eps, out[i], ldout, nullptr, 0, stream);
+    else if (!tall) st = fm_scale_cast_bf16(G[i], dtype, rows, cols, ldg, sumsq, eps, X + i * mk, K, XT + i * mk, M, stream);
+    else            st = fm_scale_cast_bf16(G[i], dtype, rows, cols, ldg, sumsq, eps, XT + i * mk, M, X + i * mk, K, stream);
+    if (st) return st;
+  }
+  if (steps == 0) return FM_OK;
+
+  bf16_t* A = reinterpret_cast<bf16_t*>(w + l.a);
+  bf16_t* P = reinterpret_cast<bf16_t*>(w + l.p);
+  float* pdiag = reinterpret_cast<float*>(w + l.pdiag);   // diagonal of P, kept in fp32
+  for (int s = 0; s < steps; ++s) {
+    const bool last = s + 1 == steps;
+    bf16_t* Xn = reinterpret_cast<bf16_t*>(w + l.x[(s + 1) & 1]);
+    bf16_t* XTn = reinterpret_cast<bf16_t*>(w + l.xt[(s + 1) & 1]);
+    GemmArgs g = {};
+    // A = X X^T
+    g.A = g.B = X; g.lda = g.ldb = K; g.bs_a = g.bs_b = mk;
+    g.C = g.C2 = A; g.c_rs = g.c2_rs = M; g.c_cs = g.c2_cs = 1; g.bs_c = g.bs_c2 = mm;
+    g.Ma = g.Nb = M; g.Kc = K; g.beta = 1.0f; g.symmetric = 1; g.batch = batch;
+    if (launch_gemm_nt(g, gws, gws_bytes, hs)) return FM_ERR_LAUNCH;
+    // P = b A + c A A, diagonal in fp32
+    g = GemmArgs{};
+    g.A = g.B = g.E = g.ET = A; g.lda = g.ldb = g.lde = g.ldet = M;
+    g.bs_a = g.bs_b = g.bs_e = g.bs_et = mm;
+    g.C = g.C2 = P; g.c_rs = g.c2_rs = M; g.c_cs = g.c2_cs = 1; g.bs_c = g.bs_c2 = mm;
+    g.Ma = g.Nb = g.Kc = M; g.alpha = b; g.beta = c; g.symmetric = 1; g.batch = batch;
+    g.diag_out = pdiag; g.bs_do = (int64_t)l.pdiag_stride;
+    if (launch_gemm_nt(g, gws, gws_bytes, hs)) return FM_ERR_LAUNCH;
+    // X' = (a + diag) X + P X, and its transpose; the last step writes the caller's orientation only
+    g = GemmArgs{};
+    g.A = P; g.lda = M; g.bs_a = mm;
+    g.B = g.ET = XT; g.ldb = g.ldet = M; g.bs_b = g.bs_et = mk;
+    g.E = X; g.lde = K; g.bs_e = mk;
+    g.Ma = M; g.Nb = K; g.Kc = M; g.alpha = a; g.beta = 1.0f; g.symmetric = 0; g.batch = batch;
+    g.row_alpha = pdiag; g.bs_ra = (int64_t)l.pdiag_stride;
+    g.c_cs = g.c2_cs = 1;
+    if (!last) {
+      g.C = Xn; g.c_rs = K; g.bs_c = mk;
+      g.C2 = XTn; g.c2_rs = M; g.bs_c2 = mk;
+    } else if (!tall) {   // the result has G's shape: X itself
+      g.C = static_cast<bf16_t*>(out[0]); g.c_rs = ldout; g.use_c_list = 1;
+      for (int i = 0; i < batch; ++i) g.c_list[i] = static_cast<bf16_t*>(out[i]);
+    } else {              // or its transpose
+      g.C2 = static_cast<bf16_t*>(out[0]); g.c2_rs = ldout; g.use_c2_list = 1;
+      for (int i = 0; i < batch; ++i) g.c2_list[i] = static_cast<bf16_t*>(out[i]);
+    }
+    if (launch_gemm_nt(g, gws, gws_bytes, hs)) return FM_ERR_LAUNCH;
+    X = Xn; XT = XTn;
+  }
+  return FM_OK;
 }
 
 int fm_newtonschulz_bf16(const void* G, int dtype, int rows, int cols, int64_t ldg, void* out,
                          int64_t ldout, int steps, float a, float b, float c, float eps, void* ws,
                          size_t ws_bytes, fm_stream_t stream) {
-  if (bad_dtype(dtype)) return FM_ERR_DTYPE;
-  if (rows < 0 || cols < 0 || steps < 0) return FM_ERR_SHAPE;
-  if (rows == 0 || cols == 0) return FM_OK;
-  if (!G || !out) return FM_ERR_NULL;
-  if (ldg < cols || ldout < cols) return FM_ERR_STRIDE;
-  if (misaligned(G, dtype_size(dtype)) || misaligned(out, 2)) return FM_ERR_ALIGN;
-  if (overlaps(mat_range(G, rows, cols, ldg, dtype_size(dtype)), mat_range(out, rows, cols, ldout, 2)))
-    return FM_ERR_ALIAS;
-  const NsLayout l = ns_layout(rows, cols);
-  if (!ws || ws_bytes < l.total) return FM_ERR_WORKSPACE;
-  if (reinterpret_cast<uintptr_t>(ws) % 256 != 0) return FM_ERR_ALIGN;
-
-  unsigned char* w = static_cast<unsigned char*>(ws);
-  float* sumsq = reinterpret_cast<float*>(w + l.sumsq);
-  void* partials = w + l.partials;
-  void* gws = w + l.gemm;
-  const size_t gws_bytes = l.total - l.gemm;
-  const bool tall = rows > cols;
-  const int M = tall ? cols : rows, K = tall ? rows : cols;
-
-  int st = fm_sumsq(G, dtype, rows, cols, ldg, sumsq, partials, fm_sumsq_workspace_bytes(), stream);
-  if (st) return st;
-
-  // The iteration runs on X (M x K) with M <= K.  G is X when it is wide and X^T when it is
-  // tall, so the scaled cast of G is X in one case and X^T in the other.
-  void* X = w + l.x[0];
-  void* XT = w + l.xt[0];
-  if (steps == 0) return fm_scale_cast_bf16(G, dtype, rows, cols, ldg, sumsq, eps, out, ldout, nullptr, 0, stream);
-  if (!tall) st = fm_scale_cast_bf16(G, dtype, rows, cols, ldg, sumsq, eps, X, K, XT, M, stream);
-  else       st = fm_scale_cast_bf16(G, dtype, rows, cols, ldg, sumsq, eps, XT, M, X, K, stream);
-  if (st) return st;
-
-  void* A = w + l.a;
-  void* P = w + l.p;
-  float* pdiag = reinterpret_cast<float*>(w + l.pdiag);   // diagonal of P, kept in fp32
-  for (int s = 0; s < steps; ++s) {
-    const bool last = s + 1 == steps;
-    st = fm_syrk_bf16(X, K, A, M, 1, M, K, gws, gws_bytes, stream);
-    if (st) return st;
-    st = fm_syrk_poly_bf16(A, M, P, M, M, b, c, pdiag, gws, gws_bytes, stream);
-    if (st) return st;
-    void* Xn = w + l.x[(s + 1) & 1];
-    void* XTn = w + l.xt[(s + 1) & 1];
-    if (!last)
-      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, Xn, K, XTn, M, M, K, a, pdiag, gws, gws_bytes, stream);
-    else if (!tall)   // the result has G's shape: X itself
-      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, out, ldout, nullptr, 0, M, K, a, pdiag, gws, gws_bytes, stream);
-    else              // or its transpose
-      st = fm_gemm_axpby_bf16(P, M, XT, M, X, K, nullptr, 0, out, ldout, M, K, a, pdiag, gws, gws_bytes, stream);
-    if (st) return st;
-    X = Xn; XT = XTn;
-  }
-  return FM_OK;
+  const void* gs[1] = {G};
+  void* os[1] = {out};
+  if (rows > 0 && cols > 0 && (!G || !out)) return FM_ERR_NULL;
+  return fm_newtonschulz_batched_bf16(gs, dtype, 1, rows, cols, ldg, os, ldout, steps, a, b, c, eps,
+                                      ws, ws_bytes, stream);
 }
 
 int fm_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,

@@ -81,7 +81,8 @@ __device__ __forceinline__ unsigned short f2bf(float v) {
 __device__ __forceinline__ float bf2f(bf16_t v) { return (float)v; }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArgs p) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArgs pb) {
+  const GemmArgs p = batch_view(pb, (int)blockIdx.y);
   constexpr int NT = 64 * WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -216,8 +217,8 @@ template <int BM, int BN, int WAVES_M, int WAVES_N>
 static int launch_cfg(GemmArgs a, bool aligned, hipStream_t stream) {
   a.tiles_m = (a.Ma + BM - 1) / BM;
   a.tiles_n = (a.Nb + BN - 1) / BN;
-  a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;
-  dim3 grid((unsigned)a.num_tiles), block(64 * WAVES_M * WAVES_N);
+  a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;   // per matrix here
+  dim3 grid((unsigned)a.num_tiles, (unsigned)a.batch), block(64 * WAVES_M * WAVES_N);
   if (aligned)
     hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true>), grid, block, 0, stream, a);
   else
@@ -232,12 +233,13 @@ int launch_gemm_general(GemmArgs a, hipStream_t stream) {
   // Large outputs take 256x256 tiles (8 waves, 128x64 per wave); small ones take 128x128 tiles
   // (4 waves, 64x64 per wave) so that more workgroups exist than the chip has CUs.
   const int64_t big_tiles = (int64_t)((a.Ma + 255) / 256) * ((a.Nb + 255) / 256);
-  const int64_t work_tiles = a.symmetric ? (big_tiles + (a.Ma + 255) / 256) / 2 : big_tiles;
+  const int64_t work_tiles = (a.symmetric ? (big_tiles + (a.Ma + 255) / 256) / 2 : big_tiles) * a.batch;
   if (work_tiles >= 256) return launch_cfg<256, 256, 2, 4>(a, aligned, stream);
   return launch_cfg<128, 128, 2, 2>(a, aligned, stream);
 }
 
 int launch_gemm_nt(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
+  if (a.batch < 1) a.batch = 1;
   if (gemm_fast_eligible(a) && ws && ws_bytes >= gemm_fast_workspace_bytes(a.Ma, a.Nb, a.symmetric != 0))
     return launch_gemm_fast(a, ws, ws_bytes, stream);
   return launch_gemm_general(a, stream);

@@ -299,8 +299,11 @@ struct FastArgs {
 // the blocks, row-major inside a block; blocks below the diagonal are skipped and blocks on it are
 // triangles when the product is symmetric), so the ~32 tiles an XCD works on at any one time touch
 // about 8 + 8 operand panels instead of one panel per tile, and its L2 serves most of the copies.
-__device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& ti, int& tj) {
+__device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& b, int& ti, int& tj) {
   constexpr int SB = 8;
+  const int per_matrix = g.num_tiles / g.batch;
+  b = pos / per_matrix;
+  pos -= b * per_matrix;
   const int nbm = (g.tiles_m + SB - 1) / SB, nbn = (g.tiles_n + SB - 1) / SB;
   for (int I = 0; I < nbm; ++I) {
     const int rows = (g.tiles_m - I * SB) < SB ? (g.tiles_m - I * SB) : SB;
@@ -330,7 +333,6 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   unsigned char* const sA1 = smem + 2 * OPER_BYTES;
   unsigned char* const sB1 = smem + 3 * OPER_BYTES;
 
-  const GemmArgs& g = p.g;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -366,8 +368,9 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     }
     const int n = ke - kb;
 
-    int ti, tj;
-    tile_at(g, pos, ti, tj);
+    int bi, ti, tj;
+    tile_at(p.g, pos, bi, ti, tj);
+    const GemmArgs g = batch_view(p.g, bi);
     const int m0 = ti * BM, n0 = tj * BN;
 
     // DMA copy q of this wave fills LDS rows (q*4 + wave)*8 .. +8 of an operand stage (the output
@@ -462,12 +465,13 @@ __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int t = blockIdx.x >> 3, blk = (blockIdx.x >> 1) & 3, h = blockIdx.x & 1;
-  int ti, tj;
-  tile_at(p.g, p.rounds * p.grid + t, ti, tj);
+  int bi, ti, tj;
+  tile_at(p.g, p.rounds * p.grid + t, bi, ti, tj);
+  const GemmArgs g = batch_view(p.g, bi);
   sum_parts_to_stage(p.partials + (size_t)t * p.split * PART_FLOATS + (blk * 2 + h) * (128 * 64), p.split, stg,
                      lane, wave * 8, wave * 8 + 8);
   __syncthreads();
-  epilogue_half(p.g, stg, ti, tj, blk >> 1, blk & 1, h, lane, wave * 4, wave * 4 + 4);
+  epilogue_half(g, stg, ti, tj, blk >> 1, blk & 1, h, lane, wave * 4, wave * 4 + 4);
 }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -507,11 +511,16 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   if (a.C2 && (a.c2_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C2) & 15))) return false;
   if (a.E && a.C && (a.lde % 8 != 0 || (reinterpret_cast<uintptr_t>(a.E) & 15))) return false;
   if (a.E && a.C2 && (!a.ET || a.ldet % 8 != 0 || (reinterpret_cast<uintptr_t>(a.ET) & 15))) return false;
-  if (a.row_alpha && (reinterpret_cast<uintptr_t>(a.row_alpha) & 15)) return false;
+  if (a.row_alpha && ((reinterpret_cast<uintptr_t>(a.row_alpha) & 15) || a.bs_ra % 4 != 0)) return false;
+  for (int i = 0; i < a.batch && i < kMaxBatch; ++i) {
+    if (a.use_c_list && (reinterpret_cast<uintptr_t>(a.c_list[i]) & 15)) return false;
+    if (a.use_c2_list && (reinterpret_cast<uintptr_t>(a.c2_list[i]) & 15)) return false;
+  }
+  if (a.batch > 1 && (a.bs_a % 8 || a.bs_b % 8 || a.bs_e % 8 || a.bs_et % 8 || a.bs_c % 8 || a.bs_c2 % 8)) return false;
   // small problems: 128x128 tiles fill the chip better than few 256x256 tiles
   // (FLASHMUON_FAST_MIN_UNITS overrides the threshold, e.g. 0 to exercise this path on small inputs)
   const long long tm = a.Ma / BM, tn = a.Nb / BN;
-  const long long tiles = a.symmetric ? tm * (tm + 1) / 2 : tm * tn;
+  const long long tiles = (a.symmetric ? tm * (tm + 1) / 2 : tm * tn) * (a.batch < 1 ? 1 : a.batch);
   static const long long min_units = [] {
     const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS");
     return e ? std::atoll(e) : 8192LL;
@@ -528,7 +537,8 @@ size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric) {
 int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
   a.tiles_m = a.Ma / BM;
   a.tiles_n = a.Nb / BN;
-  a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;
+  if (a.batch < 1) a.batch = 1;
+  a.num_tiles = (a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n) * a.batch;
   FastArgs f;
   f.g = a;
   f.nk = a.Kc / BKF;

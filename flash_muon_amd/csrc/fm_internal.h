@@ -11,6 +11,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
+constexpr int kMaxBatch = 8;          // matrices per batched launch
+
 // Arguments of the one NT contraction every GEMM-shaped kernel here is an instance of:
 //     acc[i][j] = sum_k A[i][k] * B[j][k]            (A: Ma x Kc, B: Nb x Kc, k contiguous)
 //     v         = E ? (alpha + row_alpha[i]) * E[i][j] + beta * acc : acc   (row_alpha optional)
@@ -30,9 +32,31 @@ struct GemmArgs {
   const float* row_alpha;   // optional per-row addition to alpha
   float* diag_out;          // optional fp32 copy of the diagonal, which is then stored as zero
   int symmetric;
-  int tiles_m, tiles_n;   // number of block tiles along each output dimension
-  int num_tiles;          // tiles actually computed (triangular count when symmetric)
+  // `batch` independent problems of the same shape in one launch: matrix b of an operand starts
+  // b * stride elements after matrix 0 (strides of absent operands are ignored)
+  int batch;
+  int64_t bs_a, bs_b, bs_e, bs_et, bs_c, bs_c2, bs_ra, bs_do;
+  // outputs that are not evenly spaced: when set, matrix b writes to c_list[b] / c2_list[b]
+  int use_c_list, use_c2_list;
+  bf16_t* c_list[kMaxBatch];
+  bf16_t* c2_list[kMaxBatch];
+  int tiles_m, tiles_n;   // number of block tiles along each output dimension of one matrix
+  int num_tiles;          // tiles actually computed, over the whole batch
 };
+
+// the arguments of matrix b of a batch, as a single-matrix problem
+__host__ __device__ inline GemmArgs batch_view(const GemmArgs& g, int b) {
+  GemmArgs v = g;
+  v.A += b * g.bs_a;
+  v.B += b * g.bs_b;
+  if (v.E) v.E += b * g.bs_e;
+  if (v.ET) v.ET += b * g.bs_et;
+  if (g.use_c_list) v.C = g.c_list[b]; else if (v.C) v.C += b * g.bs_c;
+  if (g.use_c2_list) v.C2 = g.c2_list[b]; else if (v.C2) v.C2 += b * g.bs_c2;
+  if (v.row_alpha) v.row_alpha += b * g.bs_ra;
+  if (v.diag_out) v.diag_out += b * g.bs_do;
+  return v;
+}
 
 // Enqueue the contraction described by `args` on `stream`, on the 256x256 stream-K path when the
 // shape, the alignment and the workspace allow it and on the general tiled path otherwise.

@@ -6,6 +6,8 @@ fm_newtonschulz_bf16; the momentum and weight updates (muon.py:99-100, 87-89) ar
 each.  The all-gather of muon.py:108 has no counterpart: only world_size == 1 is implemented,
 and no process group is needed.
 """
+import ctypes
+
 import torch
 from torch import Tensor
 
@@ -24,19 +26,26 @@ def _rows_unit_stride(G):
     return G.contiguous()
 
 
-def _newtonschulz_into(G, out, steps):
-    """Orthogonalise 2-D G (bf16/fp16/fp32, rows unit-stride) into `out` (bf16, same shape)."""
-    rows, cols = G.shape
+MAX_BATCH = 8   # kMaxBatch of the library: matrices per batched launch
+
+
+def _newtonschulz_into(Gs, outs, steps):
+    """Orthogonalise the 2-D matrices Gs (one shape, dtype and row pitch; bf16/fp16/fp32, rows
+    unit-stride) into `outs` (bf16, same shape, one row pitch), every stage one launch for all."""
+    G0, n = Gs[0], len(Gs)
+    rows, cols = G0.shape
     lib = _lib.load()
     a, b, c = NS_COEFFS
-    ldg = G.stride(0) if rows > 1 else cols
-    ldo = out.stride(0) if rows > 1 else cols
-    with torch.cuda.device(G.device):
-        ws, ws_bytes = _lib.workspace(lib.fm_newtonschulz_workspace_bytes(rows, cols), G.device)
-        st = lib.fm_newtonschulz_bf16(G.data_ptr(), _lib.dtype_code(G.dtype), rows, cols, ldg,
-                                      out.data_ptr(), ldo, steps, a, b, c, NS_EPS,
-                                      ws.data_ptr(), ws_bytes, _lib.stream_ptr(G.device))
-    _lib.check("fm_newtonschulz_bf16", st)
+    ldg = G0.stride(0) if rows > 1 else cols
+    ldo = outs[0].stride(0) if rows > 1 else cols
+    g_ptrs = (ctypes.c_void_p * n)(*[g.data_ptr() for g in Gs])
+    o_ptrs = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    with torch.cuda.device(G0.device):
+        ws, ws_bytes = _lib.workspace(lib.fm_newtonschulz_batched_workspace_bytes(n, rows, cols), G0.device)
+        st = lib.fm_newtonschulz_batched_bf16(g_ptrs, _lib.dtype_code(G0.dtype), n, rows, cols, ldg,
+                                              o_ptrs, ldo, steps, a, b, c, NS_EPS,
+                                              ws.data_ptr(), ws_bytes, _lib.stream_ptr(G0.device))
+    _lib.check("fm_newtonschulz_batched_bf16", st)
 
 
 def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
@@ -61,7 +70,7 @@ def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
         return fast_newtonschulz(G.mT, steps).mT
     G = _rows_unit_stride(G)
     out = torch.empty(G.shape, dtype=torch.bfloat16, device=G.device)
-    _newtonschulz_into(G, out, int(steps))
+    _newtonschulz_into([G], [out], int(steps))
     return out
 
 
@@ -77,19 +86,23 @@ class Muon(torch.optim.Optimizer):
         nesterov: Whether to use Nesterov-style momentum in the internal SGD. (recommended)
         ns_steps: The number of Newton-Schulz iteration steps to use.
         rank, world_size: required, as in the reference; only (0, 1) is implemented.
+        batch: (not in the reference) how many same-shape matrices are orthogonalised per launch,
+            1..8; default 8.
 
     Not for embeddings, the final fully connected layer or 0/1-D parameters; 4-D convolution
     filters are flattened over their last three dimensions.
     """
 
     def __init__(self, params, lr=0.02, weight_decay=0.01, momentum=0.95, nesterov=True, ns_steps=5,
-                 rank=None, world_size=None):
+                 rank=None, world_size=None, batch=None):
         if (rank is None) or (world_size is None):
             raise Exception("world_size and rank params required, if you want to use this optimizer on a single GPU, pass rank=0 and world_size=1.")
         if world_size != 1 or rank != 0:
             raise NotImplementedError("this build implements the single-GPU step only: pass rank=0 and world_size=1")
         self.rank = rank
         self.world_size = world_size
+        self.batch = MAX_BATCH if batch is None else max(1, min(int(batch), MAX_BATCH))
+        self._staging = {}
         defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum, nesterov=nesterov, ns_steps=ns_steps)
         params = [*params]
         param_groups = []
@@ -109,41 +122,64 @@ class Muon(torch.optim.Optimizer):
         for group in self.param_groups:
             update: Tensor = group["update_buffer_views"][self.rank]
             lr, wd, mu = group["lr"], group["weight_decay"], group["momentum"]
+            nesterov = bool(group["nesterov"])
+            # The matrices of one shape and dtype are independent (flash_muon/muon.py:90-103 walks
+            # them one by one): take them `batch` at a time so that each Newton-Schulz stage is one
+            # launch over the whole batch.
+            buckets = {}
             for p in group["params"]:
                 g = p.grad
                 assert g is not None
                 assert p.is_cuda and g.is_cuda, "Muon parameters and gradients must be CUDA tensors"
-                state = self.state[p]
-                if "momentum_buffer" not in state:
-                    state["momentum_buffer"] = torch.zeros_like(g, memory_format=torch.contiguous_format)
-                buf: Tensor = state["momentum_buffer"]
-                if not buf.is_contiguous():   # e.g. a state loaded from elsewhere
-                    buf = state["momentum_buffer"] = buf.contiguous()
+                buckets.setdefault((tuple(g.shape), g.dtype, g.device), []).append(p)
+            for (_, _, dev), plist in buckets.items():
+                staging = self._staging_rows(update.numel(), min(self.batch, len(plist)), dev)
+                for i0 in range(0, len(plist), self.batch):
+                    chunk = plist[i0:i0 + self.batch]
+                    srcs = []
+                    stream = _lib.stream_ptr(dev)
+                    for p in chunk:
+                        g = p.grad
+                        state = self.state[p]
+                        if "momentum_buffer" not in state:
+                            state["momentum_buffer"] = torch.zeros_like(g, memory_format=torch.contiguous_format)
+                        buf: Tensor = state["momentum_buffer"]
+                        if not buf.is_contiguous():   # e.g. a state loaded from elsewhere
+                            buf = state["momentum_buffer"] = buf.contiguous()
+                        # buf.lerp_(g, 1 - mu); g.lerp_(buf, mu) in place on p.grad (muon.py:99-100)
+                        gc = g if g.is_contiguous() else g.contiguous()
+                        with torch.cuda.device(dev):
+                            st = lib.fm_momentum_nesterov(gc.data_ptr(), buf.data_ptr(), _lib.dtype_code(gc.dtype),
+                                                          gc.numel(), 1 - mu, mu, 1 if nesterov else 0, stream)
+                        _lib.check("fm_momentum_nesterov", st)
+                        if gc is not g and nesterov:
+                            g.copy_(gc)
+                        src = gc if nesterov else buf
+                        if src.ndim == 4:   # conv filters (muon.py:101-102)
+                            src = src.view(len(src), -1)
+                        assert src.ndim == 2, "Input `d_in` must be a 2D tensor"
+                        srcs.append(src)
+                    # orthogonalise (muon.py:103) into rows of the staging buffer
+                    outs = [staging[i].view(srcs[i].shape) for i in range(len(chunk))]
+                    _newtonschulz_into(srcs, outs, group["ns_steps"])
+                    # p *= 1 - lr*wd ; p += -lr*sqrt(max(1, rows/cols)) * update (muon.py:87-89)
+                    for i, p in enumerate(chunk):
+                        pc = p if p.is_contiguous() else p.contiguous()
+                        alpha = -lr * max(1, p.size(-2) / p.size(-1)) ** 0.5
+                        with torch.cuda.device(dev):
+                            st = lib.fm_weight_update(pc.data_ptr(), _lib.dtype_code(pc.dtype), staging[i].data_ptr(),
+                                                      pc.numel(), 1 - lr * wd, alpha, stream)
+                        _lib.check("fm_weight_update", st)
+                        if pc is not p:
+                            p.copy_(pc)
+                    last = staging[len(chunk) - 1]
+                # the group's update buffer ends up holding the last update, as in muon.py:108
+                update.copy_(last)
 
-                # buf.lerp_(g, 1 - mu); g.lerp_(buf, mu) in place on p.grad (muon.py:99-100)
-                gc = g if g.is_contiguous() else g.contiguous()
-                code = _lib.dtype_code(gc.dtype)
-                stream = _lib.stream_ptr(gc.device)
-                with torch.cuda.device(gc.device):
-                    st = lib.fm_momentum_nesterov(gc.data_ptr(), buf.data_ptr(), code, gc.numel(),
-                                                  1 - mu, mu, 1 if group["nesterov"] else 0, stream)
-                _lib.check("fm_momentum_nesterov", st)
-                if gc is not g and group["nesterov"]:
-                    g.copy_(gc)
-                src = gc if group["nesterov"] else buf
-                if src.ndim == 4:   # conv filters (muon.py:101-102)
-                    src = src.view(len(src), -1)
-                assert src.ndim == 2, "Input `d_in` must be a 2D tensor"
-
-                # orthogonalise straight into the group's update buffer (muon.py:103, 108)
-                _newtonschulz_into(src, update.view(src.shape), group["ns_steps"])
-
-                # p *= 1 - lr*wd ; p += -lr*sqrt(max(1, rows/cols)) * update (muon.py:87-89)
-                pc = p if p.is_contiguous() else p.contiguous()
-                alpha = -lr * max(1, p.size(-2) / p.size(-1)) ** 0.5
-                with torch.cuda.device(pc.device):
-                    st = lib.fm_weight_update(pc.data_ptr(), _lib.dtype_code(pc.dtype), update.data_ptr(),
-                                              pc.numel(), 1 - lr * wd, alpha, stream)
-                _lib.check("fm_weight_update", st)
-                if pc is not p:
-                    p.copy_(pc)
+    def _staging_rows(self, numel, rows, device):
+        """[rows, numel] bf16 scratch the batched orthogonalisation writes its updates to."""
+        key = (numel, str(device))
+        t = self._staging.get(key)
+        if t is None or t.size(0) < rows:
+            t = self._staging[key] = torch.empty(rows, numel, dtype=torch.bfloat16, device=device)
+        return t

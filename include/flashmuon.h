@@ -131,6 +131,20 @@ FM_API int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int6
  * Replaces fast_newtonschulz: flash_muon/muon.py:6-33.
  */
 FM_API size_t fm_newtonschulz_workspace_bytes(int rows, int cols);
+
+/* ---------------------------------------------------------------------------------------------
+ * The same for `batch` (1..8) matrices of one shape and dtype, with every GEMM-shaped stage run
+ * as ONE launch over the whole batch, so that shapes whose tile count does not fill the chip
+ * (M = 4096 gives 136 tiles for 256 CUs) are packed together.  G and out are HOST arrays of
+ * `batch` device pointers; all inputs share ldg and all outputs ldout.  No out[i] may overlap
+ * any G[j] or another out[j].  This is how the step over the same-shape parameters of
+ * flash_muon/muon.py:90-103 is meant to call the path.
+ */
+FM_API size_t fm_newtonschulz_batched_workspace_bytes(int batch, int rows, int cols);
+FM_API int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int rows, int cols,
+                                        int64_t ldg, void* const* out, int64_t ldout, int steps,
+                                        float a, float b, float c, float eps,
+                                        void* ws, size_t ws_bytes, fm_stream_t stream);
 FM_API int fm_newtonschulz_bf16(const void* G, int dtype, int rows, int cols, int64_t ldg,
                          void* out, int64_t ldout, int steps, float a, float b, float c, float eps,
                          void* ws, size_t ws_bytes, fm_stream_t stream);

@@ -132,3 +132,23 @@ def test_groups_state_dict_and_missing_grad():
     params[0].grad = None
     with pytest.raises(AssertionError):
         opt.step()
+
+
+def test_batched_step_matches_unbatched():
+    """Same-shape parameters are orthogonalised several per launch; the step must not depend on it
+    beyond the fp32 summation order of split tiles."""
+    shapes = [(256, 512)] * 5 + [(512, 256)] * 3 + [(128, 1024)] * 2   # one numel, three shapes
+    ps, gs = _make(shapes, 11)
+    res = {}
+    for batch in (1, 4, 8):
+        params = _device_params(ps, gs)
+        opt = Muon(params, lr=LR, momentum=MU, rank=0, world_size=1, batch=batch)
+        opt.step()
+        opt.step()
+        res[batch] = [q.data.cpu().float() for q in params]
+        ref_p, _, ref_b, _ = oracle.muon_step(ps, gs, [None] * len(ps), LR, WD, MU, True, 5)
+        ref_p2, _, _, _ = oracle.muon_step(ref_p, gs, ref_b, LR, WD, MU, True, 5)
+        # (the second step reuses the first step's Nesterov-updated gradient, as the device does)
+    for batch in (4, 8):
+        for x, y in zip(res[1], res[batch]):
+            assert oracle.rel_fro(x, y) < 2e-3

@@ -107,3 +107,35 @@ def test_singular_values_land_in_band():
     sv = torch.linalg.svdvals(out)
     # the leading singular values (the spike and the bulk above ~1e-3 of the norm) end near 1
     assert sv[0] < 1.3 and sv[:8].min() > 0.5
+
+
+@pytest.mark.parametrize("rows,cols", [(256, 768), (640, 256), (200, 333)])
+def test_batched_matches_single_and_oracle(lib, rows, cols):
+    """One launch per stage over several matrices of a shape (fm_newtonschulz_batched_bf16): every
+    matrix meets the oracle at the same tolerance as alone, and a batch of one is the single call."""
+    import ctypes
+    from flash_muon_amd import _lib
+    Gs = [synthetic.gradient_like_bf16(rows, cols, 4, 40 + i).to(DEV) for i in range(5)]
+    outs = [torch.empty(rows, cols, dtype=torch.bfloat16, device=DEV) for _ in Gs]
+    a, b, c = oracle.NS_COEFFS
+    n = len(Gs)
+    ws = torch.empty(lib.fm_newtonschulz_batched_workspace_bytes(n, rows, cols), dtype=torch.uint8, device=DEV)
+    st = lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * n)(*[g.data_ptr() for g in Gs]), 0, n, rows, cols, cols,
+                                          (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs]), cols, 5, a, b, c, 1e-7,
+                                          ws.data_ptr(), ws.numel(), _lib.stream_ptr(Gs[0].device))
+    assert st == 0
+    for G, out in zip(Gs, outs):
+        single = fast_newtonschulz(G, 5)
+        ref = oracle.newtonschulz(G.cpu(), 5)
+        assert oracle.rel_fro(out, ref) < TOL
+        # the batch changes which tiles fall into the split last round, hence fp32 summation order
+        assert oracle.rel_fro(out, single.float()) < TOL
+    # too many matrices, a missing pointer and an output aliasing another input are refused
+    assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 9)(), 0, 9, rows, cols, cols, (ctypes.c_void_p * 9)(), cols,
+                                            5, a, b, c, 1e-7, ws.data_ptr(), ws.numel(), None) == 2
+    assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 2)(Gs[0].data_ptr(), None), 0, 2, rows, cols, cols,
+                                            (ctypes.c_void_p * 2)(outs[0].data_ptr(), outs[1].data_ptr()), cols,
+                                            5, a, b, c, 1e-7, ws.data_ptr(), ws.numel(), None) == 1
+    assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 2)(Gs[0].data_ptr(), Gs[1].data_ptr()), 0, 2, rows, cols, cols,
+                                            (ctypes.c_void_p * 2)(outs[0].data_ptr(), Gs[0].data_ptr()), cols,
+                                            5, a, b, c, 1e-7, ws.data_ptr(), ws.numel(), None) == 5
