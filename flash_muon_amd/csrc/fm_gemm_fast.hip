@@ -9,6 +9,7 @@
 // part per workgroup, so that the last round is as short as its share of the work; the parts go to
 // memory as fp32 and a second, small kernel adds them in part order and runs the epilogue.
 #include "fm_internal.h"
+#include <cstdio>
 #include <cstdlib>
 
 namespace fm {
@@ -104,41 +105,72 @@ __device__ __forceinline__ float bfbits2f(unsigned short h) {
 }
 
 
-// ---- staging of one half (64 rows x 128 columns) of a wave's accumulators in LDS -----------------
-constexpr int STG_PITCH = 68;                          // floats per column: 64 rows + 4 of padding
-constexpr int STG_WAVE_FLOATS = 128 * STG_PITCH;       // 34816 bytes per wave
-constexpr int SMEM_BYTES = 4 * STG_WAVE_FLOATS * 4;    // 139264 >= the 131072 of the operand stages
+// ---- the part of a tile after the main loop -----------------------------------------------------
+// Each wave finishes its 128x128 block a quarter (32 rows x 128 columns, one row of MFMA tiles) at
+// a time, in its own LDS region:
+//   F  fp32 accumulators of the quarter, column-major (F[c][r], 4-row groups XOR-swizzled by c/8):
+//      written 16 bytes per lane straight from the accumulator layout, read without serious bank
+//      conflicts by both passes below;
+//   E  the epilogue operand of the quarter (bf16, row-major), two buffers, brought in by the DMA
+//      form of global_load while the previous quarter is being written out;
+//   RA the per-row additions to alpha of the block's 128 rows.
+// Nothing is loaded from global memory between the stores of a tile: a load issued after a store
+// has to wait for that store as well (one counter tracks both), and a loop of load-compute-store
+// then runs at one memory round trip per iteration.
+constexpr int QF_PITCH = 36;                              // floats per column: 32 rows + 4 of padding
+constexpr int QF_FLOATS = 128 * QF_PITCH;                 // 18432 bytes
+constexpr int QE_BYTES = 32 * 256;                        // one E buffer: 32 rows of 128 bf16
+constexpr int EPI_WAVE_BYTES = QF_FLOATS * 4 + 2 * QE_BYTES + 512;   // 35328
+constexpr int QUARTER_FLOATS = 128 * 32;                  // fp32 values of a quarter (partial tiles)
+constexpr int SMEM_BYTES = 4 * EPI_WAVE_BYTES;            // 141312 >= the 131072 of the operand stages
 
-// float index of row r (0..63) of column c (0..127): 4-row groups are XOR-swizzled with c/8
-__device__ __forceinline__ int stg_idx(int c, int r) { return c * STG_PITCH + (r ^ (((c >> 3) & 15) << 2)); }
-
-__device__ __forceinline__ void stage_store(const f32x16_t (&acc)[4][4], int h, float* stg, int lane) {
-  const int c = lane & 31, rg = 4 * (lane >> 5);
-#pragma unroll
-  for (int ii = 0; ii < 2; ++ii)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int i = 2 * h + ii;
-        f32x4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-        *reinterpret_cast<f32x4_t*>(stg + stg_idx(32 * j + c, 32 * ii + 8 * q + rg)) = v;
-      }
+struct EpiLds {
+  float* F;
+  unsigned char* E[2];
+  float* RA;
+  uint32_t e_addr[2];   // LDS byte addresses of the E buffers, for the DMA
+};
+__device__ __forceinline__ EpiLds epi_lds(unsigned char* wave_base) {
+  EpiLds l;
+  l.F = reinterpret_cast<float*>(wave_base);
+  l.E[0] = wave_base + QF_FLOATS * 4;
+  l.E[1] = l.E[0] + QE_BYTES;
+  l.RA = reinterpret_cast<float*>(l.E[1] + QE_BYTES);
+  l.e_addr[0] = FM_LDS_ADDR(l.E[0]);
+  l.e_addr[1] = FM_LDS_ADDR(l.E[1]);
+  return l;
 }
 
-// the 128 x 64 floats of the staged half, in staging order, to a partial-tile slot (coalesced)
-__device__ __forceinline__ void copy_stage_to_ws(const float* stg, float* dst, int lane) {
+// float index of row r (0..31) of column c (0..127) in F
+__device__ __forceinline__ int qf_idx(int c, int r) { return c * QF_PITCH + (r ^ (((c >> 3) & 7) << 2)); }
+
+// accumulators of MFMA tile row i -> F.  Register 4q+e of lane l in MFMA tile (i, j) is row
+// 8q + 4(l/32) + e, column 32j + l%32 of the quarter: four consecutive rows of one column.
+template <int I>
+__device__ __forceinline__ void stage_store(const f32x16_t (&acc)[4][4], float* F, int lane) {
+  const int c = lane & 31, rg = 4 * (lane >> 5);
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      f32x4_t v = {acc[I][j][4 * q], acc[I][j][4 * q + 1], acc[I][j][4 * q + 2], acc[I][j][4 * q + 3]};
+      *reinterpret_cast<f32x4_t*>(F + qf_idx(32 * j + c, 8 * q + rg)) = v;
+    }
+}
+
+// the 128 x 32 floats of the staged quarter, in staging order, to a partial-tile slot (coalesced)
+__device__ __forceinline__ void copy_stage_to_ws(const float* F, float* dst, int lane) {
 #pragma unroll 8
-  for (int it = 0; it < 32; ++it) {
-    const int idx = it * 64 + lane;             // 16-byte unit: column idx/16, 4-row group idx%16
-    const f32x4_t v = *reinterpret_cast<const f32x4_t*>(stg + (idx >> 4) * STG_PITCH + (idx & 15) * 4);
+  for (int it = 0; it < 16; ++it) {
+    const int idx = it * 64 + lane;             // 16-byte unit: column idx/8, 4-row group idx%8
+    const f32x4_t v = *reinterpret_cast<const f32x4_t*>(F + (idx >> 3) * QF_PITCH + (idx & 7) * 4);
     *reinterpret_cast<f32x4_t*>(dst + idx * 4) = v;
   }
 }
 
-// sum of the `nparts` parts of one staged half, in part order, back into staging layout; this wave
-// takes the 16-byte units it_begin*64 .. it_end*64.  Loads go out eight parts at a time.
-__device__ __forceinline__ void sum_parts_to_stage(const float* parts, int nparts, float* stg, int lane,
+// sum of the `nparts` parts of one quarter, in part order, into F; this wave takes the 16-byte units
+// it_begin*64 .. it_end*64.  Loads go out eight parts at a time.
+__device__ __forceinline__ void sum_parts_to_stage(const float* parts, int nparts, float* F, int lane,
                                                    int it_begin, int it_end) {
   for (int it = it_begin; it < it_end; ++it) {
     const int idx = it * 64 + lane;
@@ -153,134 +185,118 @@ __device__ __forceinline__ void sum_parts_to_stage(const float* parts, int npart
 #pragma unroll
       for (int t = 0; t < 8; ++t) if (t0 + t < nparts) v += x[t];
     }
-    *reinterpret_cast<f32x4_t*>(stg + (idx >> 4) * STG_PITCH + (idx & 15) * 4) = v;
+    *reinterpret_cast<f32x4_t*>(F + (idx >> 3) * QF_PITCH + (idx & 7) * 4) = v;
   }
 }
 
-// value stored for accumulator a at (row, col): a itself, or al * e + beta * a; spelled with an
-// explicit multiply and fma so that the two passes below produce the same bits
-__device__ __forceinline__ float epi_value(float a, float e, float al, float beta, bool has_e) {
-  return has_e ? __builtin_fmaf(al, e, __fmul_rn(beta, a)) : a;
+// DMA of the epilogue operand of quarter q of the block (32 rows x 256 bytes) into an E buffer:
+// copies n_begin .. n_end of the 8 (4 rows each) are issued by the calling wave
+__device__ __forceinline__ void epi_dma_e(const GemmArgs& g, int row_base, int col_base, int lane,
+                                          uint32_t lds_addr, int n_begin, int n_end) {
+  const bf16_t* src = g.E + (int64_t)row_base * g.lde + col_base;
+  for (int n = n_begin; n < n_end; ++n) {
+    const uint32_t voff = (uint32_t)(((n * 4 + (lane >> 4)) * (int)g.lde + (lane & 15) * 8) * 2);
+    dma16(voff, src, lds_addr + n * 1024);
+  }
 }
 
-// Epilogue of the staged half h of the wave's block: rows m0 + wm*128 + 64h .. +64, columns
-// n0 + wn*128 .. +128.  Pass 1 writes C2 (the transposed copy) 8 rows x 1 column per lane, pass 2
-// writes C 1 row x 8 columns per lane; both 16 bytes per lane and coalesced.  HAS_E: the epilogue
-// operand is present; HAS_RA: so is the per-row addition to alpha; DIAG: this is a diagonal tile
-// of a symmetric product (masks, and the fp32 diagonal if it is asked for).
-template <bool HAS_E, bool HAS_RA, bool DIAG>
-__device__ __forceinline__ void epilogue_half_t(const GemmArgs& g, const float* stg, int ti, int tj,
-                                                int wm, int wn, int h, int lane, int it_begin, int it_end) {
-  const int row_base = ti * BM + wm * 128 + 64 * h;    // global row of staged row 0
-  const int col_base = tj * BN + wn * 128;             // global column of staged column 0
+// Epilogue of the staged quarter: rows row_base .. +32, columns col_base .. +128, iterations
+// it_begin .. it_end (of 8) of each pass.  The direct pass (passes & 1) writes C, 1 row x 8 columns
+// per lane, and when a transposed copy is wanted too puts the rounded values back into F; the
+// transposed pass (passes & 2) writes C2, 8 rows x 1 column per lane, from F.  Both store 16 bytes
+// per lane, and both copies carry the same bits.
+// HAS_E: v = (alpha + row_alpha) * E + beta * acc, else v = acc.  DIAG: a diagonal tile of a
+// symmetric product (masks, and the fp32 diagonal if it is asked for).
+template <bool HAS_E, bool DIAG>
+__device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, const unsigned char* Eb,
+                                                   const float* RA, int ra_off, int row_base, int col_base,
+                                                   int lane, int it_begin, int it_end, int passes) {
   const float alpha = g.alpha, beta = g.beta;
   const bool dout = DIAG && g.diag_out != nullptr;
-  // Iterations go four at a time, all loads of the four first: a load issued after a store has to
-  // wait for that store as well (one counter tracks both), which would serialise the loop on the
-  // write latency.
-  if (g.C2) {
-    unsigned short* C2 = reinterpret_cast<unsigned short*>(g.C2);
-    const unsigned short* ET = reinterpret_cast<const unsigned short*>(g.ET);
-    for (int it0 = it_begin; it0 < it_end; it0 += 4) {
-      f32x4_t lo[4], hi[4], r_lo[4], r_hi[4];
-      uint4 ev[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int idx = (it0 + u) * 64 + lane;
-        const int c = idx >> 3, r0 = (idx & 7) * 8;    // column c, rows r0 .. r0+7 of the staged half
-        const int col = col_base + c, row = row_base + r0;
-        lo[u] = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0));
-        hi[u] = *reinterpret_cast<const f32x4_t*>(stg + stg_idx(c, r0 + 4));
-        if (HAS_E) ev[u] = *reinterpret_cast<const uint4*>(ET + (int64_t)col * g.ldet + row);
-        if (HAS_RA) {
-          r_lo[u] = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row);
-          r_hi[u] = *reinterpret_cast<const f32x4_t*>(g.row_alpha + row + 4);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int idx = (it0 + u) * 64 + lane;
-        const int c = idx >> 3, r0 = (idx & 7) * 8;
-        const int col = col_base + c, row = row_base + r0;
-        const float a[8] = {lo[u][0], lo[u][1], lo[u][2], lo[u][3], hi[u][0], hi[u][1], hi[u][2], hi[u][3]};
-        union { uint4 v; unsigned short s[8]; } e, o;
-        if (HAS_E) e.v = ev[u];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          float al = alpha;
-          if (HAS_RA) al += (k < 4) ? r_lo[u][k & 3] : r_hi[u][k & 3];
-          float v = epi_value(a[k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al, beta, HAS_E);
-          if (dout && row + k == col) v = 0.0f;        // pass 2 hands the fp32 diagonal out
-          o.s[k] = f2bf(v);
-        }
-        unsigned short* dst = C2 + (int64_t)col * g.c2_rs + row;
-        // diagonal tile: mirror only what lies strictly above the diagonal (col > row + k); a group
-        // of 8 rows is all above it, all on or below it, or straddles it
-        if (!DIAG || col > row + 7) {
-          *reinterpret_cast<uint4*>(dst) = o.v;
-        } else if (col > row) {
-#pragma unroll
-          for (int k = 0; k < 8; ++k) if (col > row + k) dst[k] = o.s[k];
-        }
-      }
-    }
-  }
-  if (g.C) {
+  const bool has_ra = HAS_E && g.row_alpha != nullptr;
+  if ((passes & 1) && (g.C || HAS_E)) {
     unsigned short* C = reinterpret_cast<unsigned short*>(g.C);
-    const unsigned short* E = reinterpret_cast<const unsigned short*>(g.E);
-    for (int it0 = it_begin; it0 < it_end; it0 += 4) {
-      float a[4][8], ra[4];
-      uint4 ev[4];
+#pragma unroll 4
+    for (int it = it_begin; it < it_end; ++it) {
+      const int idx = it * 64 + lane;
+      const int r = idx >> 4, c0 = (idx & 15) * 8;     // row r, columns c0 .. c0+7 of the quarter
+      const int row = row_base + r, col = col_base + c0;
+      float a[8];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int idx = (it0 + u) * 64 + lane;
-        const int r = idx >> 4, c0 = (idx & 15) * 8;   // row r, columns c0 .. c0+7 of the staged half
-        const int row = row_base + r, col = col_base + c0;
+      for (int k = 0; k < 8; ++k) a[k] = F[qf_idx(c0 + k, r)];
+      union { uint4 v; unsigned short s[8]; } e, o;
+      if (HAS_E) e.v = *reinterpret_cast<const uint4*>(Eb + r * 256 + c0 * 2);
+      const float al = has_ra ? alpha + RA[ra_off + r] : alpha;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) a[u][k] = stg[stg_idx(c0 + k, r)];
-        if (HAS_E) ev[u] = *reinterpret_cast<const uint4*>(E + (int64_t)row * g.lde + col);
-        if (HAS_RA) ra[u] = g.row_alpha[row];
+      for (int k = 0; k < 8; ++k) {
+        float v = HAS_E ? __builtin_fmaf(al, bfbits2f(e.s[k]), beta * a[k]) : a[k];
+        if (dout && row == col + k) { g.diag_out[row] = v; v = 0.0f; }
+        o.s[k] = f2bf(v);
+        if (HAS_E && g.C2) F[qf_idx(c0 + k, r)] = bfbits2f(o.s[k]);   // what the transposed pass stores
       }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int idx = (it0 + u) * 64 + lane;
-        const int r = idx >> 4, c0 = (idx & 15) * 8;
-        const int row = row_base + r, col = col_base + c0;
-        union { uint4 v; unsigned short s[8]; } e, o;
-        if (HAS_E) e.v = ev[u];
-        const float al = HAS_RA ? alpha + ra[u] : alpha;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          float v = epi_value(a[u][k], HAS_E ? bfbits2f(e.s[k]) : 0.0f, al, beta, HAS_E);
-          if (dout && row == col + k) { g.diag_out[row] = v; v = 0.0f; }
-          o.s[k] = f2bf(v);
-        }
+      if (g.C) {
         unsigned short* dst = C + (int64_t)row * g.c_rs + col;
-        // diagonal tile: keep what lies on or above the diagonal (col + k >= row); the rest of the
-        // row comes from pass 1 of the mirrored position, i.e. from the same accumulator
+        // diagonal tile: keep what lies on or above the diagonal (col + k >= row); the rest of
+        // the row comes from the transposed pass of the mirrored position, the same accumulator
         if (!DIAG || col >= row) {
           *reinterpret_cast<uint4*>(dst) = o.v;
         } else if (col + 7 >= row) {
-#pragma unroll
-          for (int k = 0; k < 8; ++k) if (col + k >= row) dst[k] = o.s[k];
+          // the kept elements are the suffix k >= row - col: at most one 8-, 4- and 2-byte store
+          const int k0 = row - col;                       // 1..7
+          if (k0 <= 4) *reinterpret_cast<uint2*>(dst + 4) = make_uint2(o.v.z, o.v.w);
+          const int k1 = k0 <= 4 ? k0 : k0 - 4;           // first kept element inside the 4 left to look at
+          unsigned short* d4 = dst + (k0 <= 4 ? 0 : 4);
+          const unsigned short* s4 = o.s + (k0 <= 4 ? 0 : 4);
+          if (k1 <= 2 && k1 < 4) *reinterpret_cast<uint32_t*>(d4 + 2) = (uint32_t)s4[2] | ((uint32_t)s4[3] << 16);
+          if (k1 == 1 || k1 == 3) d4[k1] = s4[k1];
+          if (k1 == 0) *reinterpret_cast<uint32_t*>(d4) = (uint32_t)s4[0] | ((uint32_t)s4[1] << 16);
         }
+      }
+    }
+  }
+  if ((passes & 2) && g.C2) {
+    unsigned short* C2 = reinterpret_cast<unsigned short*>(g.C2);
+#pragma unroll 4
+    for (int it = it_begin; it < it_end; ++it) {
+      const int idx = it * 64 + lane;
+      const int c = idx >> 2, r0 = (idx & 3) * 8;      // column c, rows r0 .. r0+7 of the quarter
+      const int col = col_base + c, row = row_base + r0;
+      const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(F + qf_idx(c, r0));
+      const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(F + qf_idx(c, r0 + 4));
+      const float a[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      union { uint4 v; unsigned short s[8]; } o;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        float v = a[k];
+        if (!HAS_E && dout && row + k == col) v = 0.0f;
+        o.s[k] = f2bf(v);
+      }
+      unsigned short* dst = C2 + (int64_t)col * g.c2_rs + row;
+      // diagonal tile: mirror only what lies strictly above the diagonal (col > row + k); a group
+      // of 8 rows is all above it, all on or below it, or straddles it
+      if (!DIAG || col > row + 7) {
+        *reinterpret_cast<uint4*>(dst) = o.v;
+      } else if (col > row) {
+        // the kept elements are the prefix k < col - row: at most one 8-, 4- and 2-byte store
+        const int n = col - row;                          // 1..7
+        if (n >= 4) *reinterpret_cast<uint2*>(dst) = make_uint2(o.v.x, o.v.y);
+        const int b = n >= 4 ? 4 : 0, m = n - b;          // m elements left from dst[b]
+        if (m >= 2) *reinterpret_cast<uint32_t*>(dst + b) = (uint32_t)o.s[b] | ((uint32_t)o.s[b + 1] << 16);
+        if (m & 1) dst[b + (m & 2)] = o.s[b + (m & 2)];
       }
     }
   }
 }
 
-__device__ __forceinline__ void epilogue_half(const GemmArgs& g, const float* stg, int ti, int tj,
-                                              int wm, int wn, int h, int lane, int it_begin = 0, int it_end = 16) {
-  const bool diag = g.symmetric && ti == tj;
+__device__ __forceinline__ void epilogue_quarter(const GemmArgs& g, bool diag, float* F, const unsigned char* Eb,
+                                                 const float* RA, int ra_off, int row_base, int col_base,
+                                                 int lane, int it_begin, int it_end, int passes) {
   if (!g.E) {
-    if (diag) epilogue_half_t<false, false, true>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
-    else epilogue_half_t<false, false, false>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
-  } else if (diag) {
-    epilogue_half_t<true, false, true>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
-  } else if (g.row_alpha) {
-    epilogue_half_t<true, true, false>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+    if (diag) epilogue_quarter_t<false, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+    else epilogue_quarter_t<false, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
   } else {
-    epilogue_half_t<true, false, false>(g, stg, ti, tj, wm, wn, h, lane, it_begin, it_end);
+    if (diag) epilogue_quarter_t<true, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+    else epilogue_quarter_t<true, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
   }
 }
 
@@ -293,7 +309,16 @@ struct FastArgs {
   int rem;              // tiles of the last, partial round
   int split;            // k parts per tile of the last round (1: whole tiles, nothing to add up)
   int dbg;              // tuning aid: bit 0 skips the epilogue, bit 1 skips the main loop
+  int stagger_ticks;    // start delay per XCD index, in 10 ns ticks of the constant-rate clock
+#ifdef FM_TIMING
+  long long* stamps;    // timing build only: cycle stamps of workgroup 0, wave 0
+#endif
 };
+#ifdef FM_TIMING
+#define FM_STAMP(i) if (tid == 0 && ((i) == 0 || (i) == 2 || (i) == 7)) p.stamps[(blockIdx.x * 4 + round) * 4 + ((i) == 0 ? 0 : (i) == 2 ? 1 : 2)] = wall_clock64();
+#else
+#define FM_STAMP(i)
+#endif
 
 // Position in the schedule -> tile coordinates.  Tiles are visited in 8x8 blocks (row-major over
 // the blocks, row-major inside a block; blocks below the diagonal are skipped and blocks on it are
@@ -340,7 +365,16 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous block of positions
   // so that the tiles it holds at any one time are neighbours in the blocked tile order.
   int w = (int)blockIdx.x;
-  if (p.grid >= 8) w = (w & 7) * (p.grid >> 3) + (w >> 3);
+  if (p.grid >= 8) {
+    // XCD x starts x * stagger later than XCD 0 and stays that far behind: the rounds of one XCD
+    // still run in step, but the XCDs reach their epilogues (a burst of output traffic with the
+    // matrix cores idle) one after the other instead of all at once.
+    if (p.stagger_ticks > 0) {
+      const long long until = wall_clock64() + (long long)(w & 7) * p.stagger_ticks;
+      while (wall_clock64() < until) __builtin_amdgcn_s_sleep(8);
+    }
+    w = (w & 7) * (p.grid >> 3) + (w >> 3);
+  }
 
   const uint32_t lA0 = FM_LDS_ADDR(sA0) + wave * 1024, lB0 = FM_LDS_ADDR(sB0) + wave * 1024;
   const uint32_t lA1 = FM_LDS_ADDR(sA1) + wave * 1024, lB1 = FM_LDS_ADDR(sB1) + wave * 1024;
@@ -368,6 +402,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     }
     const int n = ke - kb;
 
+    FM_STAMP(0)
     int bi, ti, tj;
     tile_at(p.g, pos, bi, ti, tj);
     const GemmArgs g = batch_view(p.g, bi);
@@ -407,6 +442,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       }
       wait_vmcnt<16>();
       __syncthreads();
+      FM_STAMP(1)
       read_frags(f0, sA0, sB0, ao, bo, 0);
       // stages go through the loop in pairs (a loop with a second exit in the middle makes the
       // register allocator give up on keeping the accumulators in place); an odd last stage follows
@@ -437,41 +473,89 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       }
       wait_vmcnt<0>();
       __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
+      FM_STAMP(2)
     }
 
-    // ---- accumulators -> LDS, then everything else from LDS with plain loops --------------------
-    // Register 4q+e of lane l in MFMA tile (i, j) is row 32i + 8q + 4(l/32) + e, column 32j + l%32
-    // of the wave's 128x128 block: four consecutive rows of one column.  Each wave parks one half of
-    // its block (64 rows x 128 columns, fp32) at a time in its own LDS region, column-major
-    // (T[c][r], 4-row groups XOR-swizzled by c/8), which both passes below read without conflicts.
+    // ---- accumulators -> LDS a quarter at a time, and out (see the notes above EpiLds) -----------
     const bool split = (n != p.nk);
-    float* const stg = reinterpret_cast<float*>(smem) + wave * STG_WAVE_FLOATS;
+    const bool diag = g.symmetric && ti == tj;
+    const EpiLds L = epi_lds(smem + wave * EPI_WAVE_BYTES);
     float* const slot = p.partials + (size_t)((pos - p.rounds * p.grid) * p.split + part) * PART_FLOATS;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      stage_store(acc, h, stg, lane);
-      if (split) copy_stage_to_ws(stg, slot + (wave * 2 + h) * (128 * 64), lane);
-      else if (!(p.dbg & 1)) epilogue_half(g, stg, ti, tj, wm, wn, h, lane);
+    const int row0 = m0 + wm * 128, col0 = n0 + wn * 128;
+    const bool use_e = !split && g.E != nullptr;
+    if (use_e) {
+      epi_dma_e(g, row0, col0, lane, L.e_addr[0], 0, 8);
+      if (g.row_alpha) {   // the block's 128 rows, before any store of this tile
+        const float2 ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+        *reinterpret_cast<float2*>(L.RA + lane * 2) = ra;
+      }
     }
+    // The wait for quarter q's operand must not wait for the stores of quarter q-1, which were
+    // issued after its copies: it allows as many operations in flight as are known to follow them
+    // (8 copies of the next operand, 8 stores per output written; fewer on a diagonal tile, whose
+    // masked stores are not counted on).
+#define FM_QUARTER(q)                                                                                  \
+    {                                                                                                  \
+      if (use_e && q < 3) epi_dma_e(g, row0 + 32 * (q + 1), col0, lane, L.e_addr[(q + 1) & 1], 0, 8);  \
+      stage_store<q>(acc, L.F, lane);                                                                  \
+      if (split) {                                                                                     \
+        copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);                           \
+      } else if (!(p.dbg & 1)) {                                                                       \
+        if (use_e) {                                                                                   \
+          const int later = (q < 3 ? 8 : 0);                                                           \
+          const int stores = (q == 0 || diag) ? 0 : ((g.C ? 8 : 0) + (g.C2 ? 8 : 0));                  \
+          if (later + stores >= 24) wait_vmcnt<24>();                                                  \
+          else if (later + stores >= 16) wait_vmcnt<16>();                                             \
+          else if (later + stores >= 8) wait_vmcnt<8>();                                               \
+          else wait_vmcnt<0>();                                                                        \
+        }                                                                                              \
+        epilogue_quarter(g, diag, L.F, L.E[q & 1], L.RA, 32 * q, row0 + 32 * q, col0, lane, 0, 8, 3);  \
+      }                                                                                                \
+    }
+    FM_QUARTER(0)
+    FM_STAMP(3)
+    FM_QUARTER(1)
+    FM_STAMP(4)
+    FM_QUARTER(2)
+    FM_STAMP(5)
+    FM_QUARTER(3)
+    FM_STAMP(6)
+#undef FM_QUARTER
     __syncthreads();   // the next tile's copies land in the memory the staging just used
+    FM_STAMP(7)
   }
 }
 
-// Second kernel of a split last round: one workgroup per (tail tile, 128x128 block, half).  Its four
-// waves add the parts in part order, so the bits do not depend on which workgroup finished when,
-// into one staging buffer, and then share the iterations of the same epilogue the main kernel runs.
+// Second kernel of a split last round: one workgroup per (tail tile, 128x128 block, quarter).  Its
+// four waves add the parts in part order, so the bits do not depend on which workgroup finished
+// when, into one staging buffer, and then share the iterations of the same epilogue the main kernel
+// runs.
 __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
-  __shared__ __align__(16) float stg[STG_WAVE_FLOATS];
+  __shared__ __align__(1024) unsigned char smem[EPI_WAVE_BYTES];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int t = blockIdx.x >> 3, blk = (blockIdx.x >> 1) & 3, h = blockIdx.x & 1;
+  const int t = blockIdx.x >> 4, blk = (blockIdx.x >> 2) & 3, q = blockIdx.x & 3;
   int bi, ti, tj;
   tile_at(p.g, p.rounds * p.grid + t, bi, ti, tj);
   const GemmArgs g = batch_view(p.g, bi);
-  sum_parts_to_stage(p.partials + (size_t)t * p.split * PART_FLOATS + (blk * 2 + h) * (128 * 64), p.split, stg,
-                     lane, wave * 8, wave * 8 + 8);
+  const EpiLds L = epi_lds(smem);
+  const int row0 = ti * BM + (blk >> 1) * 128, col0 = tj * BN + (blk & 1) * 128;
+  if (g.E) {
+    epi_dma_e(g, row0 + 32 * q, col0, lane, L.e_addr[0], wave * 2, wave * 2 + 2);
+    if (g.row_alpha && wave == 0) {
+      const float2 ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+      *reinterpret_cast<float2*>(L.RA + lane * 2) = ra;
+    }
+  }
+  sum_parts_to_stage(p.partials + (size_t)t * p.split * PART_FLOATS + (blk * 4 + q) * QUARTER_FLOATS, p.split, L.F,
+                     lane, wave * 4, wave * 4 + 4);
+  wait_vmcnt<0>();
   __syncthreads();
-  epilogue_half(g, stg, ti, tj, blk >> 1, blk & 1, h, lane, wave * 4, wave * 4 + 4);
+  const bool diag = g.symmetric && ti == tj;
+  // direct pass, then (after everybody has put its rounded values back) the transposed pass
+  epilogue_quarter(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 1);
+  __syncthreads();
+  epilogue_quarter(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 2);
 }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -545,11 +629,33 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   fast_schedule(a.num_tiles, f.nk, f);
   f.dbg = 0;
   if (const char* e = std::getenv("FLASHMUON_DBG")) f.dbg = std::atoi(e);
+#ifdef FM_TIMING
+  static long long* stamps = nullptr;
+  if (!stamps) { (void)hipMalloc(&stamps, 256 * 16 * 8); (void)hipMemset(stamps, 0, 256 * 16 * 8); }
+  f.stamps = stamps;
+  {
+    static long long h[256 * 16];
+    static int calls = 0;
+    (void)hipMemcpy(h, stamps, sizeof(h), hipMemcpyDeviceToHost);   // stamps of the previous launch
+    if (h[0] && ++calls == 20) {
+      long long t0 = h[0];
+      for (int b = 0; b < 256; ++b) if (h[b * 16] && h[b * 16] < t0) t0 = h[b * 16];
+      for (int b = 0; b < 256; ++b) {
+        fprintf(stderr, "wg %3d xcd %d:", b, b & 7);
+        for (int r = 0; r < 3; ++r)
+          fprintf(stderr, "  [%lld %lld %lld]", h[(b * 4 + r) * 4] - t0, h[(b * 4 + r) * 4 + 1] - t0, h[(b * 4 + r) * 4 + 2] - t0);
+        fprintf(stderr, "\n");
+      }
+    }
+  }
+#endif
+  f.stagger_ticks = 0;
+  if (const char* e = std::getenv("FLASHMUON_STAGGER_US")) f.stagger_ticks = (int)(std::atof(e) * 100.0);
   f.partials = static_cast<float*>(ws);
   if (f.split > 1 && (!ws || ws_bytes < (size_t)f.rem * f.split * PART_FLOATS * sizeof(float))) return -1;
   hipLaunchKernelGGL(gemm_nt_rounds_kernel, dim3(f.grid), dim3(256), 0, stream, f);
   if (f.split > 1)
-    hipLaunchKernelGGL(gemm_nt_reduce_kernel, dim3(f.rem * 8), dim3(256), 0, stream, f);
+    hipLaunchKernelGGL(gemm_nt_reduce_kernel, dim3(f.rem * 16), dim3(256), 0, stream, f);
   return (int)hipGetLastError();
 }
 
