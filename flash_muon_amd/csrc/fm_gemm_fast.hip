@@ -9,7 +9,6 @@
 // part per workgroup, so that the last round is as short as its share of the work; the parts go to
 // memory as fp32 and a second, small kernel adds them in part order and runs the epilogue.
 #include "fm_internal.h"
-#include <cstdio>
 #include <cstdlib>
 
 namespace fm {
@@ -308,17 +307,7 @@ struct FastArgs {
   int rounds;           // full rounds: tiles [0, rounds * grid) are computed whole
   int rem;              // tiles of the last, partial round
   int split;            // k parts per tile of the last round (1: whole tiles, nothing to add up)
-  int dbg;              // tuning aid: bit 0 skips the epilogue, bit 1 skips the main loop
-  int stagger_ticks;    // start delay per XCD index, in 10 ns ticks of the constant-rate clock
-#ifdef FM_TIMING
-  long long* stamps;    // timing build only: cycle stamps of workgroup 0, wave 0
-#endif
 };
-#ifdef FM_TIMING
-#define FM_STAMP(i) if (tid == 0 && ((i) == 0 || (i) == 2 || (i) == 7)) p.stamps[(blockIdx.x * 4 + round) * 4 + ((i) == 0 ? 0 : (i) == 2 ? 1 : 2)] = wall_clock64();
-#else
-#define FM_STAMP(i)
-#endif
 
 // Position in the schedule -> tile coordinates.  Tiles are visited in 8x8 blocks (row-major over
 // the blocks, row-major inside a block; blocks below the diagonal are skipped and blocks on it are
@@ -365,16 +354,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous block of positions
   // so that the tiles it holds at any one time are neighbours in the blocked tile order.
   int w = (int)blockIdx.x;
-  if (p.grid >= 8) {
-    // XCD x starts x * stagger later than XCD 0 and stays that far behind: the rounds of one XCD
-    // still run in step, but the XCDs reach their epilogues (a burst of output traffic with the
-    // matrix cores idle) one after the other instead of all at once.
-    if (p.stagger_ticks > 0) {
-      const long long until = wall_clock64() + (long long)(w & 7) * p.stagger_ticks;
-      while (wall_clock64() < until) __builtin_amdgcn_s_sleep(8);
-    }
-    w = (w & 7) * (p.grid >> 3) + (w >> 3);
-  }
+  if (p.grid >= 8) w = (w & 7) * (p.grid >> 3) + (w >> 3);
 
   const uint32_t lA0 = FM_LDS_ADDR(sA0) + wave * 1024, lB0 = FM_LDS_ADDR(sB0) + wave * 1024;
   const uint32_t lA1 = FM_LDS_ADDR(sA1) + wave * 1024, lB1 = FM_LDS_ADDR(sB1) + wave * 1024;
@@ -401,8 +381,6 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       ke = (int)((long long)p.nk * (part + 1) / p.split);
     }
     const int n = ke - kb;
-
-    FM_STAMP(0)
     int bi, ti, tj;
     tile_at(p.g, pos, bi, ti, tj);
     const GemmArgs g = batch_view(p.g, bi);
@@ -442,12 +420,10 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       }
       wait_vmcnt<16>();
       __syncthreads();
-      FM_STAMP(1)
       read_frags(f0, sA0, sB0, ao, bo, 0);
       // stages go through the loop in pairs (a loop with a second exit in the middle makes the
       // register allocator give up on keeping the accumulators in place); an odd last stage follows
       int it = 0;
-      if (p.dbg & 2) it = n & ~1;
       for (; it + 2 <= n; it += 2) {
         phase(acc, f0, f1, sA0, sB0, ao, bo, 1);
         phase(acc, f1, f0, sA0, sB0, ao, bo, 2);
@@ -473,7 +449,6 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       }
       wait_vmcnt<0>();
       __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
-      FM_STAMP(2)
     }
 
     // ---- accumulators -> LDS a quarter at a time, and out (see the notes above EpiLds) -----------
@@ -500,7 +475,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       stage_store<q>(acc, L.F, lane);                                                                  \
       if (split) {                                                                                     \
         copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);                           \
-      } else if (!(p.dbg & 1)) {                                                                       \
+      } else {                                                                       \
         if (use_e) {                                                                                   \
           const int later = (q < 3 ? 8 : 0);                                                           \
           const int stores = (q == 0 || diag) ? 0 : ((g.C ? 8 : 0) + (g.C2 ? 8 : 0));                  \
@@ -513,16 +488,11 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       }                                                                                                \
     }
     FM_QUARTER(0)
-    FM_STAMP(3)
     FM_QUARTER(1)
-    FM_STAMP(4)
     FM_QUARTER(2)
-    FM_STAMP(5)
     FM_QUARTER(3)
-    FM_STAMP(6)
 #undef FM_QUARTER
     __syncthreads();   // the next tile's copies land in the memory the staging just used
-    FM_STAMP(7)
   }
 }
 
@@ -627,30 +597,6 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   f.g = a;
   f.nk = a.Kc / BKF;
   fast_schedule(a.num_tiles, f.nk, f);
-  f.dbg = 0;
-  if (const char* e = std::getenv("FLASHMUON_DBG")) f.dbg = std::atoi(e);
-#ifdef FM_TIMING
-  static long long* stamps = nullptr;
-  if (!stamps) { (void)hipMalloc(&stamps, 256 * 16 * 8); (void)hipMemset(stamps, 0, 256 * 16 * 8); }
-  f.stamps = stamps;
-  {
-    static long long h[256 * 16];
-    static int calls = 0;
-    (void)hipMemcpy(h, stamps, sizeof(h), hipMemcpyDeviceToHost);   // stamps of the previous launch
-    if (h[0] && ++calls == 20) {
-      long long t0 = h[0];
-      for (int b = 0; b < 256; ++b) if (h[b * 16] && h[b * 16] < t0) t0 = h[b * 16];
-      for (int b = 0; b < 256; ++b) {
-        fprintf(stderr, "wg %3d xcd %d:", b, b & 7);
-        for (int r = 0; r < 3; ++r)
-          fprintf(stderr, "  [%lld %lld %lld]", h[(b * 4 + r) * 4] - t0, h[(b * 4 + r) * 4 + 1] - t0, h[(b * 4 + r) * 4 + 2] - t0);
-        fprintf(stderr, "\n");
-      }
-    }
-  }
-#endif
-  f.stagger_ticks = 0;
-  if (const char* e = std::getenv("FLASHMUON_STAGGER_US")) f.stagger_ticks = (int)(std::atof(e) * 100.0);
   f.partials = static_cast<float*>(ws);
   if (f.split > 1 && (!ws || ws_bytes < (size_t)f.rem * f.split * PART_FLOATS * sizeof(float))) return -1;
   hipLaunchKernelGGL(gemm_nt_rounds_kernel, dim3(f.grid), dim3(256), 0, stream, f);
