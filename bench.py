@@ -64,6 +64,22 @@ def _cpu_baseline(X, torch):
                       "os.cpu_count()=%d" % (M, K, reps, dt, os.cpu_count())}
 
 
+def _torch_ns(G, steps, torch):
+    """The plain-torch Newton-Schulz the reference benchmarks against (benchmark.py:23-47), on the GPU:
+    vendor GEMMs and eager elementwise ops, bf16."""
+    a, b, c = 3.4445, -4.7750, 2.0315
+    X = G.bfloat16()
+    tall = G.size(0) > G.size(1)
+    if tall:
+        X = X.T
+    X = X / (X.norm() + 1e-7)
+    for _ in range(steps):
+        A = X @ X.T
+        B = b * A + c * A @ A
+        X = a * X + B @ X
+    return X.T if tall else X
+
+
 def _extras(Xd, steps, warmup, torch):
     from flash_muon_amd import Muon, fast_newtonschulz, synthetic
     ex = {}
@@ -84,6 +100,9 @@ def _extras(Xd, steps, warmup, torch):
         fl = synthetic.ns_useful_flop(rows, cols, 5)
         ex["ns5_%dx%d_ms" % (rows, cols)] = ms
         ex["ns5_%dx%d_useful_tflops" % (rows, cols)] = fl / ms / 1e9
+        ref_ms = _time_gpu(lambda: _torch_ns(G, 5, torch), 10, 3, torch)
+        ex["torch_ns5_%dx%d_ms" % (rows, cols)] = ref_ms
+        ex["ns5_%dx%d_speedup_vs_torch" % (rows, cols)] = ref_ms / ms
         del G
     # Muon.step on Llama-7B shapes: 32 layers x (4 x 4096^2, 2 x 11008x4096, 1 x 4096x11008)
     g = torch.Generator(device="cuda").manual_seed(5)

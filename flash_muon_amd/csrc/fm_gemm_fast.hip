@@ -19,6 +19,8 @@ constexpr int BM = 256, BN = 256, BKF = 64;
 constexpr int ROWB = BKF * 2;               // bytes per LDS row
 constexpr int OPER_BYTES = BM * ROWB;       // one operand stage: 32 KiB
 constexpr int PART_FLOATS = BM * BN;        // one fp32 partial tile
+constexpr int kMaxParts = 64;               // parts one tile can be cut into
+constexpr int kMaxSlots = 768;              // partial-tile slots the workspace holds (192 MiB)
 
 #define FM_LDS_ADDR(p) ((uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(p)))
 
@@ -167,10 +169,11 @@ __device__ __forceinline__ void copy_stage_to_ws(const float* F, float* dst, int
   }
 }
 
-// sum of the `nparts` parts of one quarter, in part order, into F; this wave takes the 16-byte units
+// sum of the `nparts` parts of one quarter (slot numbers in `slots`, in k order) into F, added in that
+// order; `parts` points at the quarter inside slot 0; this wave takes the 16-byte units
 // it_begin*64 .. it_end*64.  Loads go out eight parts at a time.
-__device__ __forceinline__ void sum_parts_to_stage(const float* parts, int nparts, float* F, int lane,
-                                                   int it_begin, int it_end) {
+__device__ __forceinline__ void sum_parts_to_stage(const float* parts, const int* slots, int nparts, float* F,
+                                                   int lane, int it_begin, int it_end) {
   for (int it = it_begin; it < it_end; ++it) {
     const int idx = it * 64 + lane;
     f32x4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -179,7 +182,7 @@ __device__ __forceinline__ void sum_parts_to_stage(const float* parts, int npart
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const int tt = (t0 + t < nparts) ? t0 + t : nparts - 1;   // clamped; the value is dropped below
-        x[t] = *reinterpret_cast<const f32x4_t*>(parts + (size_t)tt * PART_FLOATS + idx * 4);
+        x[t] = *reinterpret_cast<const f32x4_t*>(parts + (size_t)slots[tt] * PART_FLOATS + idx * 4);
       }
 #pragma unroll
       for (int t = 0; t < 8; ++t) if (t0 + t < nparts) v += x[t];
@@ -299,15 +302,31 @@ __device__ __forceinline__ void epilogue_quarter(const GemmArgs& g, bool diag, f
   }
 }
 
+// The schedule works on items: item i is base part i % ksplit of tile i / ksplit, where every tile's
+// k range is cut into `ksplit` equal base parts (1 unless there are too few tiles to fill the chip
+// and k is long).  Items [0, rounds * grid) run one per workgroup in `rounds` full rounds; the `rem`
+// items left over are cut once more into `split` sub-parts each, one per workgroup, in a last round.
+// Anything that is not a whole tile is written to a partial-tile slot: item i of a full round to
+// slot i, sub-part q of left-over item j to slot tail_slot0 + j * split + q.
 struct FastArgs {
   GemmArgs g;
-  float* partials;      // rem * split fp32 tiles: part q of tail tile t is slot t * split + q
+  float* partials;      // fp32 partial tiles
   int nk;               // k stages per tile
   int grid;             // workgroups launched (a multiple of 8, or fewer than 8)
-  int rounds;           // full rounds: tiles [0, rounds * grid) are computed whole
-  int rem;              // tiles of the last, partial round
-  int split;            // k parts per tile of the last round (1: whole tiles, nothing to add up)
+  int ksplit;           // base parts per tile
+  int rounds;           // full rounds of items
+  int rem;              // items of the last, partial round
+  int split;            // sub-parts per item of the last round
+  int tail_slot0;       // first slot of the last round's sub-parts
+  int reduce_tile0;     // first tile the second kernel has to finish
 };
+
+// k stages [kb, ke) of base part `part` of `parts`, or of its sub-part `sub` of `subs`
+__device__ __forceinline__ void item_range(int nk, int part, int parts, int sub, int subs, int& kb, int& ke) {
+  const int b0 = (int)((long long)nk * part / parts), b1 = (int)((long long)nk * (part + 1) / parts);
+  kb = b0 + (int)((long long)(b1 - b0) * sub / subs);
+  ke = b0 + (int)((long long)(b1 - b0) * (sub + 1) / subs);
+}
 
 // Position in the schedule -> tile coordinates.  Tiles are visited in 8x8 blocks (row-major over
 // the blocks, row-major inside a block; blocks below the diagonal are skipped and blocks on it are
@@ -370,16 +389,19 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   }
 
   for (int round = 0; round <= p.rounds; ++round) {
-    int pos, kb, ke, part = 0;
+    int item, slot_id, kb, ke;
     if (round < p.rounds) {
-      pos = round * p.grid + w; kb = 0; ke = p.nk;
+      item = round * p.grid + w;
+      slot_id = item;
+      item_range(p.nk, item % p.ksplit, p.ksplit, 0, 1, kb, ke);
     } else {
       if (w >= p.rem * p.split) break;
-      pos = p.rounds * p.grid + w / p.split;
-      part = w - (w / p.split) * p.split;
-      kb = (int)((long long)p.nk * part / p.split);
-      ke = (int)((long long)p.nk * (part + 1) / p.split);
+      const int j = w / p.split, sub = w - j * p.split;
+      item = p.rounds * p.grid + j;
+      slot_id = p.tail_slot0 + w;
+      item_range(p.nk, item % p.ksplit, p.ksplit, sub, p.split, kb, ke);
     }
+    const int pos = item / p.ksplit;
     const int n = ke - kb;
     int bi, ti, tj;
     tile_at(p.g, pos, bi, ti, tj);
@@ -455,7 +477,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     const bool split = (n != p.nk);
     const bool diag = g.symmetric && ti == tj;
     const EpiLds L = epi_lds(smem + wave * EPI_WAVE_BYTES);
-    float* const slot = p.partials + (size_t)((pos - p.rounds * p.grid) * p.split + part) * PART_FLOATS;
+    float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
     const int row0 = m0 + wm * 128, col0 = n0 + wn * 128;
     const bool use_e = !split && g.E != nullptr;
     if (use_e) {
@@ -496,17 +518,18 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   }
 }
 
-// Second kernel of a split last round: one workgroup per (tail tile, 128x128 block, quarter).  Its
-// four waves add the parts in part order, so the bits do not depend on which workgroup finished
-// when, into one staging buffer, and then share the iterations of the same epilogue the main kernel
-// runs.
+// Second kernel, for the tiles that were not computed whole: one workgroup per (tile, 128x128
+// block, quarter).  Its four waves add the tile's parts in k order, so the bits do not depend on
+// which workgroup finished when, into one staging buffer, and then share the iterations of the
+// same epilogue the main kernel runs.
 __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
   __shared__ __align__(1024) unsigned char smem[EPI_WAVE_BYTES];
+  __shared__ int s_slot[kMaxParts];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int t = blockIdx.x >> 4, blk = (blockIdx.x >> 2) & 3, q = blockIdx.x & 3;
+  const int t = p.reduce_tile0 + (int)(blockIdx.x >> 4), blk = (blockIdx.x >> 2) & 3, q = blockIdx.x & 3;
   int bi, ti, tj;
-  tile_at(p.g, p.rounds * p.grid + t, bi, ti, tj);
+  tile_at(p.g, t, bi, ti, tj);
   const GemmArgs g = batch_view(p.g, bi);
   const EpiLds L = epi_lds(smem);
   const int row0 = ti * BM + (blk >> 1) * 128, col0 = tj * BN + (blk & 1) * 128;
@@ -517,8 +540,21 @@ __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
       *reinterpret_cast<float2*>(L.RA + lane * 2) = ra;
     }
   }
-  sum_parts_to_stage(p.partials + (size_t)t * p.split * PART_FLOATS + (blk * 4 + q) * QUARTER_FLOATS, p.split, L.F,
-                     lane, wave * 4, wave * 4 + 4);
+  // the slots of this tile's parts, in k order
+  const int first_tail_item = p.rounds * p.grid;
+  int nparts = 0;
+  for (int part = 0; part < p.ksplit; ++part) {
+    const int item = t * p.ksplit + part;
+    if (item < first_tail_item) {
+      if (threadIdx.x == 0) s_slot[nparts] = item;
+      nparts += 1;
+    } else {
+      if ((int)threadIdx.x < p.split) s_slot[nparts + threadIdx.x] = p.tail_slot0 + (item - first_tail_item) * p.split + threadIdx.x;
+      nparts += p.split;
+    }
+  }
+  __syncthreads();
+  sum_parts_to_stage(p.partials + (blk * 4 + q) * QUARTER_FLOATS, s_slot, nparts, L.F, lane, wave * 4, wave * 4 + 4);
   wait_vmcnt<0>();
   __syncthreads();
   const bool diag = g.symmetric && ti == tj;
@@ -532,23 +568,37 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
 
-// grid, rounds, remainder and split of the schedule for `num_tiles` tiles of `nk` k stages
+// the schedule for `num_tiles` tiles of `nk` k stages
 static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
-  int grid = 256;                                   // one workgroup per CU (136 KiB of LDS each)
+  int grid = 256;                                   // one workgroup per CU (138 KiB of LDS each)
   if (const char* e = std::getenv("FLASHMUON_GRID")) grid = std::atoi(e);   // tuning aid
-  if (grid > num_tiles) grid = num_tiles;           // rem * split never exceeds the grid below
+  if (grid > 256) grid = 256;
+  // Too few tiles for one round (M = 4096 gives 136 symmetric tiles) and a long k: cut every tile
+  // in two along k, which doubles the items at the price of one fp32 round trip per tile.
+  int ksplit = 1;
+  if (num_tiles * 5 < grid * 3 && nk >= 128) ksplit = 2;
+  if (const char* e = std::getenv("FLASHMUON_KSPLIT")) ksplit = std::atoi(e);   // tuning aid
+  if (ksplit < 1 || ksplit > nk || ksplit > 4) ksplit = 1;
+  if (ksplit > 1 && (int64_t)num_tiles * ksplit + grid > kMaxSlots) ksplit = 1;   // slots: items + rem * split
+  const int items = num_tiles * ksplit;
+  if (grid > items) grid = items;                   // rem * split never exceeds the grid below
   if (grid >= 8) grid &= ~7;
   if (grid < 1) grid = 1;
   f.grid = grid;
-  f.rounds = num_tiles / grid;
-  f.rem = num_tiles % grid;
+  f.ksplit = ksplit;
+  f.rounds = items / grid;
+  f.rem = items % grid;
   f.split = 1;
   if (f.rem > 0) {
-    int s = grid / f.rem;                           // parts that fit in one round of workgroups
-    if (s > nk) s = nk;
-    if (s > 32) s = 32;                             // bounds the partial-tile traffic
+    int s = grid / f.rem;                           // sub-parts that fit in one round of workgroups
+    const int base_stages = nk / ksplit;
+    if (s > base_stages) s = base_stages;
+    if (s > 16) s = 16;                             // bounds the partial-tile traffic
     f.split = s < 1 ? 1 : s;
   }
+  f.tail_slot0 = ksplit > 1 ? f.rounds * grid : 0;
+  // whole tiles need no second kernel: with ksplit == 1 only the left-over items, if they were cut
+  f.reduce_tile0 = ksplit > 1 ? 0 : (f.split > 1 ? f.rounds * grid : num_tiles);
 }
 
 bool gemm_fast_eligible(const GemmArgs& a) {
@@ -585,7 +635,8 @@ bool gemm_fast_eligible(const GemmArgs& a) {
 
 size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric) {
   (void)Ma; (void)Nb; (void)symmetric;
-  return (size_t)256 * PART_FLOATS * sizeof(float);   // rem * split <= grid <= 256 partial tiles
+  // items of full rounds (only when tiles are cut: fewer than 2 * 256 of them) + rem * split <= 256
+  return (size_t)kMaxSlots * PART_FLOATS * sizeof(float);
 }
 
 int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
@@ -598,10 +649,14 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   f.nk = a.Kc / BKF;
   fast_schedule(a.num_tiles, f.nk, f);
   f.partials = static_cast<float*>(ws);
-  if (f.split > 1 && (!ws || ws_bytes < (size_t)f.rem * f.split * PART_FLOATS * sizeof(float))) return -1;
+  const int slots = f.tail_slot0 + f.rem * f.split;
+  const int reduce_tiles = a.num_tiles - f.reduce_tile0;
+  if (reduce_tiles > 0 && (!ws || slots > kMaxSlots || ws_bytes < (size_t)slots * PART_FLOATS * sizeof(float) ||
+                           f.ksplit * f.split > kMaxParts))
+    return -1;
   hipLaunchKernelGGL(gemm_nt_rounds_kernel, dim3(f.grid), dim3(256), 0, stream, f);
-  if (f.split > 1)
-    hipLaunchKernelGGL(gemm_nt_reduce_kernel, dim3(f.rem * 16), dim3(256), 0, stream, f);
+  if (reduce_tiles > 0)
+    hipLaunchKernelGGL(gemm_nt_reduce_kernel, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
   return (int)hipGetLastError();
 }
 

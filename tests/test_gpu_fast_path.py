@@ -1,7 +1,8 @@
-"""The 256x256 stream-K path of the GEMM-shaped kernels.  It is chosen by shape (whole 256-tiles, k a
-multiple of 64, enough k stages to share out); FLASHMUON_FAST_MIN_UNITS=0 is set here, before the
-library is loaded, so that small inputs take it too and the split-tile hand-over is exercised with
-few, many and uneven parts per tile.  Integer-valued inputs make every comparison bit-exact."""
+"""The 256x256 path of the GEMM-shaped kernels (rounds of whole tiles, tiles cut along k where the
+chip would otherwise idle).  It is chosen by shape (whole 256-tiles, k a multiple of 64, enough k
+stages to share out); FLASHMUON_FAST_MIN_UNITS=0 is set here, before the library is loaded, so that
+small inputs take it too and the partial-tile hand-over is exercised with few, many and uneven
+parts per tile.  Integer-valued inputs make every comparison bit-exact."""
 import os
 
 os.environ["FLASHMUON_FAST_MIN_UNITS"] = "0"
@@ -42,6 +43,32 @@ def test_syrk_fast_integer_bit_exact(lib, M, K):
     assert torch.equal(Y2, Y)
 
 
+@pytest.mark.parametrize("ksplit", [1, 2, 3, 4])
+@pytest.mark.parametrize("M,K", [(256, 448), (768, 1024), (1280, 8192), (4096, 1024)])
+def test_syrk_fast_forced_base_split(lib, monkeypatch, M, K, ksplit):
+    """Every tile cut into `ksplit` base parts along k (the library reads the variable at each launch):
+    full rounds of partial tiles, a cut last round, and the second kernel over every tile."""
+    monkeypatch.setenv("FLASHMUON_KSPLIT", str(ksplit))
+    X = _ints((M, K), 7 * M + K + ksplit)
+    want = _exact(X.double() @ X.double().T)
+    Y = torch.full((M, M), 7.0, dtype=torch.bfloat16, device=DEV)
+    gpu_util.syrk(lib, X.to(DEV), Y)
+    assert torch.equal(Y.cpu(), want)
+
+
+@pytest.mark.parametrize("ksplit", [2, 3])
+def test_axpby_fast_forced_base_split(lib, monkeypatch, ksplit):
+    monkeypatch.setenv("FLASHMUON_KSPLIT", str(ksplit))
+    M, K = 768, 1536
+    P = _ints((M, M), 31 + ksplit, -1, 1)
+    X = _ints((M, K), 37 + ksplit)
+    d = torch.arange(M, dtype=torch.float32) % 3 - 1
+    want = _exact((2 + d.double())[:, None] * X.double() + P.double() @ X.double())
+    Xo, XoT = gpu_util.gemm_axpby(lib, P.to(DEV), X.to(DEV), 2.0, row_alpha=d.to(DEV))
+    assert torch.equal(Xo.cpu(), want)
+    assert torch.equal(XoT.cpu(), want.T)
+
+
 @pytest.mark.parametrize("M", [256, 512, 1024, 1536])
 def test_poly_fast_integer_bit_exact(lib, M):
     g = torch.Generator().manual_seed(M)
@@ -72,7 +99,7 @@ def test_axpby_fast_integer_bit_exact(lib, M, K):
 
 
 def test_fast_and_general_paths_agree_on_gaussian_input(lib):
-    """Same input through the stream-K path (with workspace) and the tiled path (without): both are
+    """Same input through the 256x256 path (with workspace) and the tiled path (without): both are
     one bf16 rounding of an fp32 sum, so they agree to within that rounding."""
     g = torch.Generator().manual_seed(5)
     X = torch.randn(1024, 2048, generator=g).bfloat16().to(DEV)
