@@ -204,11 +204,15 @@ __device__ __forceinline__ void epi_dma_e(const GemmArgs& g, int row_base, int c
 
 // Epilogue of the staged quarter: rows row_base .. +32, columns col_base .. +128, iterations
 // it_begin .. it_end (of 8) of each pass.  The direct pass (passes & 1) writes C, 1 row x 8 columns
-// per lane, and when a transposed copy is wanted too puts the rounded values back into F; the
-// transposed pass (passes & 2) writes C2, 8 rows x 1 column per lane, from F.  Both store 16 bytes
-// per lane, and both copies carry the same bits.
-// HAS_E: v = (alpha + row_alpha) * E + beta * acc, else v = acc.  DIAG: a diagonal tile of a
-// symmetric product (masks, and the fp32 diagonal if it is asked for).
+// per lane, and puts the rounded values back into F when an operand was added; the transposed pass
+// (passes & 2) writes C2, 8 rows x 1 column per lane, from F.  Both store 16 bytes per lane, and
+// both copies carry the same bits.
+// HAS_E: v = (alpha + row_alpha) * E + beta * acc, else v = acc.
+// DIAG: a diagonal tile of a symmetric product.  Its own mirror image lies inside the tile, and the
+// accumulators at (i, j) and (j, i) already hold the same bits: both add the same exact products
+// x_ik * x_jk in the same order, through the same dot-product datapath.  So such a tile is written
+// once, whole, by the direct pass and has no transposed pass.  The fp32 diagonal, if asked for, is
+// split off here.
 template <bool HAS_E, bool DIAG>
 __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, const unsigned char* Eb,
                                                    const float* RA, int ra_off, int row_base, int col_base,
@@ -223,40 +227,36 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
       const int idx = it * 64 + lane;
       const int r = idx >> 4, c0 = (idx & 15) * 8;     // row r, columns c0 .. c0+7 of the quarter
       const int row = row_base + r, col = col_base + c0;
-      float a[8];
+      float v[8];
 #pragma unroll
-      for (int k = 0; k < 8; ++k) a[k] = F[qf_idx(c0 + k, r)];
+      for (int k = 0; k < 8; ++k) v[k] = F[qf_idx(c0 + k, r)];
       union { uint4 v; unsigned short s[8]; } e, o;
-      if (HAS_E) e.v = *reinterpret_cast<const uint4*>(Eb + r * 256 + c0 * 2);
-      const float al = has_ra ? alpha + RA[ra_off + r] : alpha;
+      if (HAS_E) {
+        e.v = *reinterpret_cast<const uint4*>(Eb + r * 256 + c0 * 2);
+        const float al = has_ra ? alpha + RA[ra_off + r] : alpha;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = __builtin_fmaf(al, bfbits2f(e.s[k]), beta * v[k]);
+      }
+      if (DIAG) {                                       // selects only: no branch per element
+        const int kd = row - col;                       // the diagonal element of this row, if 0..7
+        float dv = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const bool on = dout && kd == k;
+          dv = on ? v[k] : dv;
+          v[k] = on ? 0.0f : v[k];
+        }
+        if (dout && (unsigned)kd < 8u) g.diag_out[row] = dv;
+      }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        float v = HAS_E ? __builtin_fmaf(al, bfbits2f(e.s[k]), beta * a[k]) : a[k];
-        if (dout && row == col + k) { g.diag_out[row] = v; v = 0.0f; }
-        o.s[k] = f2bf(v);
-        if (HAS_E && g.C2) F[qf_idx(c0 + k, r)] = bfbits2f(o.s[k]);   // what the transposed pass stores
+        o.s[k] = f2bf(v[k]);
+        if (HAS_E && !DIAG) F[qf_idx(c0 + k, r)] = bfbits2f(o.s[k]);   // what the transposed pass stores
       }
-      if (g.C) {
-        unsigned short* dst = C + (int64_t)row * g.c_rs + col;
-        // diagonal tile: keep what lies on or above the diagonal (col + k >= row); the rest of
-        // the row comes from the transposed pass of the mirrored position, the same accumulator
-        if (!DIAG || col >= row) {
-          *reinterpret_cast<uint4*>(dst) = o.v;
-        } else if (col + 7 >= row) {
-          // the kept elements are the suffix k >= row - col: at most one 8-, 4- and 2-byte store
-          const int k0 = row - col;                       // 1..7
-          if (k0 <= 4) *reinterpret_cast<uint2*>(dst + 4) = make_uint2(o.v.z, o.v.w);
-          const int k1 = k0 <= 4 ? k0 : k0 - 4;           // first kept element inside the 4 left to look at
-          unsigned short* d4 = dst + (k0 <= 4 ? 0 : 4);
-          const unsigned short* s4 = o.s + (k0 <= 4 ? 0 : 4);
-          if (k1 <= 2 && k1 < 4) *reinterpret_cast<uint32_t*>(d4 + 2) = (uint32_t)s4[2] | ((uint32_t)s4[3] << 16);
-          if (k1 == 1 || k1 == 3) d4[k1] = s4[k1];
-          if (k1 == 0) *reinterpret_cast<uint32_t*>(d4) = (uint32_t)s4[0] | ((uint32_t)s4[1] << 16);
-        }
-      }
+      if (g.C) *reinterpret_cast<uint4*>(C + (int64_t)row * g.c_rs + col) = o.v;
     }
   }
-  if ((passes & 2) && g.C2) {
+  if (!DIAG && (passes & 2) && g.C2) {
     unsigned short* C2 = reinterpret_cast<unsigned short*>(g.C2);
 #pragma unroll 4
     for (int it = it_begin; it < it_end; ++it) {
@@ -268,24 +268,8 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
       const float a[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       union { uint4 v; unsigned short s[8]; } o;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        float v = a[k];
-        if (!HAS_E && dout && row + k == col) v = 0.0f;
-        o.s[k] = f2bf(v);
-      }
-      unsigned short* dst = C2 + (int64_t)col * g.c2_rs + row;
-      // diagonal tile: mirror only what lies strictly above the diagonal (col > row + k); a group
-      // of 8 rows is all above it, all on or below it, or straddles it
-      if (!DIAG || col > row + 7) {
-        *reinterpret_cast<uint4*>(dst) = o.v;
-      } else if (col > row) {
-        // the kept elements are the prefix k < col - row: at most one 8-, 4- and 2-byte store
-        const int n = col - row;                          // 1..7
-        if (n >= 4) *reinterpret_cast<uint2*>(dst) = make_uint2(o.v.x, o.v.y);
-        const int b = n >= 4 ? 4 : 0, m = n - b;          // m elements left from dst[b]
-        if (m >= 2) *reinterpret_cast<uint32_t*>(dst + b) = (uint32_t)o.s[b] | ((uint32_t)o.s[b + 1] << 16);
-        if (m & 1) dst[b + (m & 2)] = o.s[b + (m & 2)];
-      }
+      for (int k = 0; k < 8; ++k) o.s[k] = f2bf(a[k]);
+      *reinterpret_cast<uint4*>(C2 + (int64_t)col * g.c2_rs + row) = o.v;
     }
   }
 }
@@ -489,8 +473,8 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     }
     // The wait for quarter q's operand must not wait for the stores of quarter q-1, which were
     // issued after its copies: it allows as many operations in flight as are known to follow them
-    // (8 copies of the next operand, 8 stores per output written; fewer on a diagonal tile, whose
-    // masked stores are not counted on).
+    // (8 copies of the next operand, 8 stores per output written; a diagonal tile writes one output,
+    // and the stores of its fp32 diagonal only make the wait longer than it has to be).
 #define FM_QUARTER(q)                                                                                  \
     {                                                                                                  \
       if (use_e && q < 3) epi_dma_e(g, row0 + 32 * (q + 1), col0, lane, L.e_addr[(q + 1) & 1], 0, 8);  \
@@ -500,7 +484,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       } else {                                                                       \
         if (use_e) {                                                                                   \
           const int later = (q < 3 ? 8 : 0);                                                           \
-          const int stores = (q == 0 || diag) ? 0 : ((g.C ? 8 : 0) + (g.C2 ? 8 : 0));                  \
+          const int stores = q == 0 ? 0 : ((g.C ? 8 : 0) + (g.C2 && !diag ? 8 : 0));                  \
           if (later + stores >= 24) wait_vmcnt<24>();                                                  \
           else if (later + stores >= 16) wait_vmcnt<16>();                                             \
           else if (later + stores >= 8) wait_vmcnt<8>();                                               \
