@@ -75,8 +75,8 @@ size_t fm_gemm_workspace_bytes(int rows_out, int cols_out) {
   return gemm_fast_workspace_bytes(rows_out, cols_out, false);
 }
 
-int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
-                 void* ws, size_t ws_bytes, fm_stream_t stream) {
+static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
+                     void* ws, size_t ws_bytes, fm_stream_t stream, int f16) {
   if (M < 0 || K < 0) return FM_ERR_SHAPE;
   if (M == 0) return FM_OK;
   if (!X && K > 0) return FM_ERR_NULL;
@@ -90,8 +90,18 @@ int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t l
   a.C = a.C2 = static_cast<bf16_t*>(Y);
   a.c_rs = a.c2_rs = ldy_row; a.c_cs = a.c2_cs = ldy_col;
   a.Ma = a.Nb = M; a.Kc = K;
-  a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1;
+  a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1; a.f16 = f16;
   return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, static_cast<hipStream_t>(stream)));
+}
+
+int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
+                 void* ws, size_t ws_bytes, fm_stream_t stream) {
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, 0);
+}
+
+int fm_syrk_f16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
+                void* ws, size_t ws_bytes, fm_stream_t stream) {
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, 1);
 }
 
 int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, float b, float c,

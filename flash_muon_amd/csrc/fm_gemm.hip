@@ -1,4 +1,4 @@
-// bf16 MFMA contraction for gfx950: acc = A * B^T with both operands k-contiguous ("NT"),
+// bf16 (or fp16) MFMA contraction for gfx950: acc = A * B^T with both operands k-contiguous ("NT"),
 // fp32 accumulation in 32x32x16 MFMA tiles, LDS double buffering, fused epilogue and an
 // optional mirrored (transposed) second store.  X*X^T, b*A + c*A*A and a*X + P*X are all
 // instances of it (see GemmArgs).
@@ -75,12 +75,7 @@ struct TileLoader {
   }
 };
 
-__device__ __forceinline__ unsigned short f2bf(float v) {
-  return __builtin_bit_cast(unsigned short, (bf16_t)v);
-}
-__device__ __forceinline__ float bf2f(bf16_t v) { return (float)v; }
-
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED, bool F16>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArgs pb) {
   const GemmArgs p = batch_view(pb, (int)blockIdx.y);
   constexpr int NT = 64 * WAVES_M * WAVES_N;
@@ -165,7 +160,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_32x32x16<F16>(fa[i], fb[j], acc[i][j]);
     }
     if (more) {
       la.store(nxt, ra);
@@ -192,13 +187,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
           float v = acc[i][j][r];
           if (has_e) {
             const float al = p.row_alpha ? p.alpha + p.row_alpha[row] : p.alpha;
-            v = al * bf2f(p.E[(int64_t)row * p.lde + col]) + p.beta * v;
+            v = al * elem_to_f32<F16>(__builtin_bit_cast(unsigned short, p.E[(int64_t)row * p.lde + col])) + p.beta * v;
           }
           if (p.diag_out && row == col) {
             p.diag_out[row] = v;
             v = 0.0f;
           }
-          unsigned short h = f2bf(v);
+          unsigned short h = f32_to_elem<F16>(v);
           // On a diagonal tile only the elements on or above the diagonal are kept, and the
           // strictly-upper ones are mirrored, so the two triangles come from the same register.
           if (!diag || col >= row) {
@@ -219,10 +214,17 @@ static int launch_cfg(GemmArgs a, bool aligned, hipStream_t stream) {
   a.tiles_n = (a.Nb + BN - 1) / BN;
   a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;   // per matrix here
   dim3 grid((unsigned)a.num_tiles, (unsigned)a.batch), block(64 * WAVES_M * WAVES_N);
-  if (aligned)
-    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true>), grid, block, 0, stream, a);
-  else
-    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false>), grid, block, 0, stream, a);
+  if (a.f16) {
+    if (aligned)
+      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true, true>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false, true>), grid, block, 0, stream, a);
+  } else {
+    if (aligned)
+      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true, false>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false, false>), grid, block, 0, stream, a);
+  }
   return (int)hipGetLastError();
 }
 

@@ -1,4 +1,4 @@
-// Fast path of the bf16 NT contraction for gfx950: 256x256 output tiles, 4 waves (one per SIMD) of
+// Fast path of the bf16 (or fp16) NT contraction for gfx950: 256x256 output tiles, 4 waves (one per SIMD) of
 // 128x128 each, 64-wide k stages copied global -> LDS by the DMA form of global_load (no VGPR
 // staging), two LDS stages.
 //
@@ -48,8 +48,7 @@ __device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
   j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
 }
 
-#define FM_MFMA(i, j, FA, FB) \
-  acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FA[i], FB[j], acc[i][j], 0, 0, 0)
+#define FM_MFMA(i, j, FA, FB) acc[i][j] = mfma_32x32x16<F16>(FA[i], FB[j], acc[i][j])
 
 struct Frag { bf16x8_t a[4], b[4]; };
 
@@ -62,6 +61,7 @@ __device__ __forceinline__ void read_frags(Frag& f, const unsigned char* sa, con
 }
 
 // 16 MFMAs of one k16 substep; the 8 fragment reads of the next substep ride on the first 8.
+template <bool F16>
 __device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
                                       const unsigned char* sa, const unsigned char* sb,
                                       const uint32_t (&ao)[4], const uint32_t (&bo)[4], int ks_next) {
@@ -80,6 +80,7 @@ __device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Fr
 // Last substep of a stage.  After the barrier every wave holds its last fragments of this stage in
 // registers and the other stage has landed, so the 16 MFMAs run interleaved with the DMA that
 // refills this stage (16 copies) and with the first fragment reads of the other stage.
+template <bool F16>
 __device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
                                            const unsigned char* nsa, const unsigned char* nsb,
                                            const uint32_t (&ao)[4], const uint32_t (&bo)[4],
@@ -97,14 +98,6 @@ __device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cu
     __builtin_amdgcn_sched_barrier(0);
   }
 }
-
-__device__ __forceinline__ unsigned short f2bf(float v) {
-  return __builtin_bit_cast(unsigned short, (bf16_t)v);
-}
-__device__ __forceinline__ float bfbits2f(unsigned short h) {
-  return __builtin_bit_cast(float, (uint32_t)h << 16);
-}
-
 
 // ---- the part of a tile after the main loop -----------------------------------------------------
 // Each wave finishes its 128x128 block a quarter (32 rows x 128 columns, one row of MFMA tiles) at
@@ -213,7 +206,7 @@ __device__ __forceinline__ void epi_dma_e(const GemmArgs& g, int row_base, int c
 // x_ik * x_jk in the same order, through the same dot-product datapath.  So such a tile is written
 // once, whole, by the direct pass and has no transposed pass.  The fp32 diagonal, if asked for, is
 // split off here.
-template <bool HAS_E, bool DIAG>
+template <bool F16, bool HAS_E, bool DIAG>
 __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, const unsigned char* Eb,
                                                    const float* RA, int ra_off, int row_base, int col_base,
                                                    int lane, int it_begin, int it_end, int passes) {
@@ -235,7 +228,7 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
         e.v = *reinterpret_cast<const uint4*>(Eb + r * 256 + c0 * 2);
         const float al = has_ra ? alpha + RA[ra_off + r] : alpha;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = __builtin_fmaf(al, bfbits2f(e.s[k]), beta * v[k]);
+        for (int k = 0; k < 8; ++k) v[k] = __builtin_fmaf(al, elem_to_f32<F16>(e.s[k]), beta * v[k]);
       }
       if (DIAG) {                                       // selects only: no branch per element
         const int kd = row - col;                       // the diagonal element of this row, if 0..7
@@ -250,8 +243,8 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
       }
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        o.s[k] = f2bf(v[k]);
-        if (HAS_E && !DIAG) F[qf_idx(c0 + k, r)] = bfbits2f(o.s[k]);   // what the transposed pass stores
+        o.s[k] = f32_to_elem<F16>(v[k]);
+        if (HAS_E && !DIAG) F[qf_idx(c0 + k, r)] = elem_to_f32<F16>(o.s[k]);   // what the transposed pass stores
       }
       if (g.C) *reinterpret_cast<uint4*>(C + (int64_t)row * g.c_rs + col) = o.v;
     }
@@ -268,22 +261,25 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
       const float a[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       union { uint4 v; unsigned short s[8]; } o;
 #pragma unroll
-      for (int k = 0; k < 8; ++k) o.s[k] = f2bf(a[k]);
+      for (int k = 0; k < 8; ++k) o.s[k] = f32_to_elem<F16>(a[k]);
       *reinterpret_cast<uint4*>(C2 + (int64_t)col * g.c2_rs + row) = o.v;
     }
   }
 }
 
+template <bool F16>
 __device__ __forceinline__ void epilogue_quarter(const GemmArgs& g, bool diag, float* F, const unsigned char* Eb,
                                                  const float* RA, int ra_off, int row_base, int col_base,
                                                  int lane, int it_begin, int it_end, int passes) {
-  if (!g.E) {
-    if (diag) epilogue_quarter_t<false, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
-    else epilogue_quarter_t<false, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
-  } else {
-    if (diag) epilogue_quarter_t<true, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
-    else epilogue_quarter_t<true, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+  if constexpr (!F16) {   // fp16 problems carry no operand E
+    if (g.E) {
+      if (diag) epilogue_quarter_t<false, true, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+      else epilogue_quarter_t<false, true, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+      return;
+    }
   }
+  if (diag) epilogue_quarter_t<F16, false, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+  else epilogue_quarter_t<F16, false, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
 }
 
 // The schedule works on items: item i is base part i % ksplit of tile i / ksplit, where every tile's
@@ -341,6 +337,7 @@ __device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& b, int&
   ti = tj = 0;   // not reached for pos < num_tiles
 }
 
+template <bool F16>
 __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // two operand stages (A0 B0 A1 B1, 32 KiB each) during the main loop, the accumulator staging of
   // the four waves afterwards
@@ -431,25 +428,25 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       // register allocator give up on keeping the accumulators in place); an odd last stage follows
       int it = 0;
       for (; it + 2 <= n; it += 2) {
-        phase(acc, f0, f1, sA0, sB0, ao, bo, 1);
-        phase(acc, f1, f0, sA0, sB0, ao, bo, 2);
-        phase(acc, f0, f1, sA0, sB0, ao, bo, 3);
+        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 1);
+        phase<F16>(acc, f1, f0, sA0, sB0, ao, bo, 2);
+        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 3);
         {
           const int kn = (it + 2 < n) ? it + 2 : n - 1;
-          tail_phase(acc, f1, f0, sA1, sB1, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA0, lB0);
+          tail_phase<F16>(acc, f1, f0, sA1, sB1, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA0, lB0);
         }
-        phase(acc, f0, f1, sA1, sB1, ao, bo, 1);
-        phase(acc, f1, f0, sA1, sB1, ao, bo, 2);
-        phase(acc, f0, f1, sA1, sB1, ao, bo, 3);
+        phase<F16>(acc, f0, f1, sA1, sB1, ao, bo, 1);
+        phase<F16>(acc, f1, f0, sA1, sB1, ao, bo, 2);
+        phase<F16>(acc, f0, f1, sA1, sB1, ao, bo, 3);
         {
           const int kn = (it + 3 < n) ? it + 3 : n - 1;
-          tail_phase(acc, f1, f0, sA0, sB0, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA1, lB1);
+          tail_phase<F16>(acc, f1, f0, sA0, sB0, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA1, lB1);
         }
       }
       if (it < n) {   // one stage left: it sits in stage 0 and its first fragments are in f0
-        phase(acc, f0, f1, sA0, sB0, ao, bo, 1);
-        phase(acc, f1, f0, sA0, sB0, ao, bo, 2);
-        phase(acc, f0, f1, sA0, sB0, ao, bo, 3);
+        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 1);
+        phase<F16>(acc, f1, f0, sA0, sB0, ao, bo, 2);
+        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 3);
 #pragma unroll
         for (int q = 0; q < 16; ++q) FM_MFMA(q >> 2, q & 3, f1.a, f1.b);
       }
@@ -463,7 +460,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     const EpiLds L = epi_lds(smem + wave * EPI_WAVE_BYTES);
     float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
     const int row0 = m0 + wm * 128, col0 = n0 + wn * 128;
-    const bool use_e = !split && g.E != nullptr;
+    const bool use_e = !F16 && !split && g.E != nullptr;
     if (use_e) {
       epi_dma_e(g, row0, col0, lane, L.e_addr[0], 0, 8);
       if (g.row_alpha) {   // the block's 128 rows, before any store of this tile
@@ -490,7 +487,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
           else if (later + stores >= 8) wait_vmcnt<8>();                                               \
           else wait_vmcnt<0>();                                                                        \
         }                                                                                              \
-        epilogue_quarter(g, diag, L.F, L.E[q & 1], L.RA, 32 * q, row0 + 32 * q, col0, lane, 0, 8, 3);  \
+        epilogue_quarter<F16>(g, diag, L.F, L.E[q & 1], L.RA, 32 * q, row0 + 32 * q, col0, lane, 0, 8, 3);  \
       }                                                                                                \
     }
     FM_QUARTER(0)
@@ -506,6 +503,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
 // block, quarter).  Its four waves add the tile's parts in k order, so the bits do not depend on
 // which workgroup finished when, into one staging buffer, and then share the iterations of the
 // same epilogue the main kernel runs.
+template <bool F16>
 __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
   __shared__ __align__(1024) unsigned char smem[EPI_WAVE_BYTES];
   __shared__ int s_slot[kMaxParts];
@@ -543,9 +541,9 @@ __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
   __syncthreads();
   const bool diag = g.symmetric && ti == tj;
   // direct pass, then (after everybody has put its rounded values back) the transposed pass
-  epilogue_quarter(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 1);
+  epilogue_quarter<F16>(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 1);
   __syncthreads();
-  epilogue_quarter(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 2);
+  epilogue_quarter<F16>(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 2);
 }
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -586,6 +584,7 @@ static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
 }
 
 bool gemm_fast_eligible(const GemmArgs& a) {
+  if (a.f16 && a.E) return false;
   if (a.Kc < BKF || a.Kc % BKF != 0) return false;
   if (a.lda % 8 != 0 || a.ldb % 8 != 0) return false;
   if ((reinterpret_cast<uintptr_t>(a.A) & 15) || (reinterpret_cast<uintptr_t>(a.B) & 15)) return false;
@@ -638,9 +637,15 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   if (reduce_tiles > 0 && (!ws || slots > kMaxSlots || ws_bytes < (size_t)slots * PART_FLOATS * sizeof(float) ||
                            f.ksplit * f.split > kMaxParts))
     return -1;
-  hipLaunchKernelGGL(gemm_nt_rounds_kernel, dim3(f.grid), dim3(256), 0, stream, f);
-  if (reduce_tiles > 0)
-    hipLaunchKernelGGL(gemm_nt_reduce_kernel, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
+  if (a.f16) {
+    hipLaunchKernelGGL(gemm_nt_rounds_kernel<true>, dim3(f.grid), dim3(256), 0, stream, f);
+    if (reduce_tiles > 0)
+      hipLaunchKernelGGL(gemm_nt_reduce_kernel<true>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
+  } else {
+    hipLaunchKernelGGL(gemm_nt_rounds_kernel<false>, dim3(f.grid), dim3(256), 0, stream, f);
+    if (reduce_tiles > 0)
+      hipLaunchKernelGGL(gemm_nt_reduce_kernel<false>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
+  }
   return (int)hipGetLastError();
 }
 

@@ -8,17 +8,38 @@ namespace fm {
 
 typedef __bf16 bf16_t;
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
 constexpr int kMaxBatch = 8;          // matrices per batched launch
 
+// The GEMM kernels exist for two 16-bit element types with the same memory layout; pointers are
+// typed bf16_t in both cases and F16 says what the bits mean.
+template <bool F16>
+__device__ __forceinline__ f32x16_t mfma_32x32x16(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+// one round-to-nearest-even conversion of an fp32 result to the element type, as its bits
+template <bool F16> __device__ __forceinline__ unsigned short f32_to_elem(float v) {
+  if constexpr (F16) return __builtin_bit_cast(unsigned short, (_Float16)v);
+  else return __builtin_bit_cast(unsigned short, (bf16_t)v);
+}
+template <bool F16> __device__ __forceinline__ float elem_to_f32(unsigned short h) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, h);
+  else return __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+
 // Arguments of the one NT contraction every GEMM-shaped kernel here is an instance of:
 //     acc[i][j] = sum_k A[i][k] * B[j][k]            (A: Ma x Kc, B: Nb x Kc, k contiguous)
 //     v         = E ? (alpha + row_alpha[i]) * E[i][j] + beta * acc : acc   (row_alpha optional)
 //     if diag_out and i == j:  diag_out[i] = v (fp32) and v = 0
-//     C [i*c_rs  + j*c_cs ] = bf16(v)                (if C  != nullptr)
-//     C2[j*c2_rs + i*c2_cs] = bf16(v)                (if C2 != nullptr; the mirrored copy)
+//     C [i*c_rs  + j*c_cs ] = round(v)               (if C  != nullptr)
+//     C2[j*c2_rs + i*c2_cs] = round(v)               (if C2 != nullptr; the mirrored copy)
+// A, B, E, C and C2 hold bf16, or fp16 when `f16` is set (fp16 is served without E only).
 // With `symmetric` set, A == B, only tiles on or above the diagonal are computed and C2 == C.
 struct GemmArgs {
   const bf16_t* A;  int64_t lda;
@@ -32,6 +53,7 @@ struct GemmArgs {
   const float* row_alpha;   // optional per-row addition to alpha
   float* diag_out;          // optional fp32 copy of the diagonal, which is then stored as zero
   int symmetric;
+  int f16;                  // element type of A, B, C, C2: 0 = bf16, 1 = fp16
   // `batch` independent problems of the same shape in one launch: matrix b of an operand starts
   // b * stride elements after matrix 0 (strides of absent operands are ignored)
   int batch;

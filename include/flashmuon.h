@@ -55,21 +55,28 @@ FM_API const char* fm_version(void);
 
 /* ---------------------------------------------------------------------------------------------
  * Scratch for the three GEMM-shaped entry points below, by the shape of their OUTPUT: (M, M) for
- * fm_syrk_bf16 and fm_syrk_poly_bf16, (M, K) for fm_gemm_axpby_bf16.  It holds the fp32 partial
- * tiles and arrival counters of output tiles whose k range is split over several workgroups.
+ * fm_syrk_bf16, fm_syrk_f16 and fm_syrk_poly_bf16, (M, K) for fm_gemm_axpby_bf16.  It holds the
+ * fp32 partial tiles of output tiles whose k range is split over several workgroups.
  * The calls also run with ws == NULL (or a smaller ws) on a slower schedule that needs none.
  */
 FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
 
 /* ---------------------------------------------------------------------------------------------
  * Y = X * X^T, X is M x K bf16 (row stride ldx, unit column stride), Y is M x M bf16 with
- * arbitrary strides (ldy_row, ldy_col).  Only upper-triangular tiles are computed; every
- * off-diagonal element is written twice from the same register, so Y == Y^T bit for bit.
- * fp32 accumulation, one round-to-nearest-even to bf16.
+ * arbitrary strides (ldy_row, ldy_col).  Only tiles on or above the diagonal are computed; every
+ * tile above it is written twice, directly and mirrored, from the same accumulators, and Y == Y^T
+ * holds bit for bit.  fp32 accumulation, one round-to-nearest-even to bf16.
  * Replaces mmt_kernel + its launch: flash_muon/matmul_transpose_triton.py:20-75, 90-101.
  */
 FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
                  int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* The same product for fp16 X and Y (the reference's kernel takes its element type from the
+ * input: flash_muon/matmul_transpose_triton.py:63): fp32 accumulation, one round-to-nearest-even
+ * to fp16, same arguments and schedule.
+ */
+FM_API int fm_syrk_f16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
+                int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * P = b*A + c*(A*A) for a SYMMETRIC M x M bf16 matrix A (row stride lda).  Same triangular
