@@ -3,6 +3,7 @@
 // optional mirrored (transposed) second store.  X*X^T, b*A + c*A*A and a*X + P*X are all
 // instances of it (see GemmArgs).
 #include "fm_internal.h"
+#include <cstdlib>
 
 namespace fm {
 
@@ -244,6 +245,7 @@ int launch_gemm_nt(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
   if (a.batch < 1) a.batch = 1;
   if (gemm_fast_eligible(a) && ws && ws_bytes >= gemm_fast_workspace_bytes(a.Ma, a.Nb, a.symmetric != 0))
     return launch_gemm_fast(a, ws, ws_bytes, stream);
+  if (gemm_mid_eligible(a) && !std::getenv("FLASHMUON_NO_MID")) return launch_gemm_mid(a, stream);
   return launch_gemm_general(a, stream);
 }
 

@@ -140,8 +140,8 @@ __device__ __forceinline__ int qf_idx(int c, int r) { return c * QF_PITCH + (r ^
 
 // accumulators of MFMA tile row i -> F.  Register 4q+e of lane l in MFMA tile (i, j) is row
 // 8q + 4(l/32) + e, column 32j + l%32 of the quarter: four consecutive rows of one column.
-template <int I>
-__device__ __forceinline__ void stage_store(const f32x16_t (&acc)[4][4], float* F, int lane) {
+template <int I, int NI>
+__device__ __forceinline__ void stage_store(const f32x16_t (&acc)[NI][4], float* F, int lane) {
   const int c = lane & 31, rg = 4 * (lane >> 5);
 #pragma unroll
   for (int j = 0; j < 4; ++j)
@@ -475,7 +475,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
 #define FM_QUARTER(q)                                                                                  \
     {                                                                                                  \
       if (use_e && q < 3) epi_dma_e(g, row0 + 32 * (q + 1), col0, lane, L.e_addr[(q + 1) & 1], 0, 8);  \
-      stage_store<q>(acc, L.F, lane);                                                                  \
+      stage_store<q, 4>(acc, L.F, lane);                                                                  \
       if (split) {                                                                                     \
         copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);                           \
       } else {                                                                       \
@@ -546,6 +546,120 @@ __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
   epilogue_quarter<F16>(g, diag, L.F, L.E[0], L.RA, 32 * q, row0 + 32 * q, col0, lane, wave * 2, wave * 2 + 2, 2);
 }
 
+// ---- 128x128 tiles, one per workgroup, for problems too small for the rounds above --------------
+// Such problems are bound by latency, not by the MFMA pipe: a handful of k stages per tile and
+// fewer tiles than CUs.  So the operand ring is deep (four 32 KiB stages in flight through the same
+// global -> LDS copies) and there is one barrier per stage.  Each of the 4 waves owns 32 rows x 128
+// columns of the tile, which is exactly one quarter of the epilogue above; the operand E of that
+// quarter is fetched into LDS of its own before the main loop starts.
+constexpr int MID_T = 128;                              // tile edge
+constexpr int MID_STAGES = 4;
+constexpr int MID_OPER = MID_T * ROWB;                  // 16 KiB
+constexpr int MID_STAGE = 2 * MID_OPER;                 // A and B
+constexpr int MID_RING = MID_STAGES * MID_STAGE;        // 131072; reused by the accumulator staging
+constexpr int MID_SMEM = MID_RING + 4 * QE_BYTES;       // + one E buffer per wave = 163840
+
+template <bool F16>
+__global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
+  __shared__ __align__(1024) unsigned char smem[MID_SMEM];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // workgroups are dealt round-robin to the 8 XCDs: give each XCD a contiguous run of tiles
+  int w = (int)blockIdx.x;
+  {
+    const int chunk = (int)gridDim.x >> 3;
+    if (w < chunk * 8) w = (w & 7) * chunk + (w >> 3);
+  }
+  int bi, ti, tj;
+  tile_at(gb, w, bi, ti, tj);
+  const GemmArgs g = batch_view(gb, bi);
+  const int m0 = ti * MID_T, n0 = tj * MID_T;
+  const int nk = g.Kc / BKF;
+  const int row0 = m0 + wave * 32, col0 = n0;
+
+  // the epilogue operand and the per-row additions first: they are long there when needed
+  const bool use_e = !F16 && g.E != nullptr;
+  unsigned char* const e_buf = smem + MID_RING + wave * QE_BYTES;
+  float ra = 0.0f;
+  if (use_e) {
+    epi_dma_e(g, row0, col0, lane, FM_LDS_ADDR(e_buf), 0, 8);
+    if (g.row_alpha) ra = g.row_alpha[row0 + (lane & 31)];
+  }
+
+  // copy q of this wave fills LDS rows (q*4 + wave)*8 .. +8 of an operand stage
+  uint32_t voA[4], voB[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int row = (q * 4 + wave) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz(row);
+    voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
+    voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
+  }
+  const bf16_t* gA = g.A + (int64_t)m0 * g.lda;
+  const bf16_t* gB = g.B + (int64_t)n0 * g.ldb;
+  const uint32_t ring = FM_LDS_ADDR(smem) + wave * 1024;
+  auto issue = [&](int stage, int slot) {   // 8 copies per wave
+    const uint32_t base = ring + slot * MID_STAGE;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dma16(voA[q], gA + stage * BKF, base + q * 4096);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) dma16(voB[q], gB + stage * BKF, base + MID_OPER + q * 4096);
+  };
+
+  // fragment offsets inside an operand stage (row = lane % 32, k half = lane / 32)
+  uint32_t ao, bo[4];
+  {
+    const int r = wave * 32 + (lane & 31);
+    ao = (uint32_t)(r * ROWB + (((lane >> 5) ^ swz(r)) << 4));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int rb = j * 32 + (lane & 31);
+      bo[j] = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
+    }
+  }
+
+  f32x16_t acc[1][4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][j][r] = 0.0f;
+
+  // Stages past the end are the last stage again (into a slot nobody reads), so that the number of
+  // copies in flight is the same at every wait.
+#pragma unroll
+  for (int s = 0; s < MID_STAGES - 1; ++s) issue(s < nk ? s : nk - 1, s);
+  for (int s = 0; s < nk; ++s) {
+    wait_vmcnt<8 * (MID_STAGES - 2)>();   // my copies of stage s have landed ...
+    __syncthreads();                      // ... and everybody's; stage s-1 is read out everywhere
+    {
+      const int nx = s + MID_STAGES - 1;
+      issue(nx < nk ? nx : nk - 1, nx & (MID_STAGES - 1));
+    }
+    const unsigned char* sa = smem + (s & (MID_STAGES - 1)) * MID_STAGE;
+    const unsigned char* sb = sa + MID_OPER;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(sa + (ao ^ (ks << 5)));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(sb + (bo[j] ^ (ks << 5)));
+        acc[0][j] = mfma_32x32x16<F16>(fa, fb, acc[0][j]);
+      }
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();   // no copy in flight and no wave still reading: the ring is free
+
+  // one quarter per wave: accumulators -> LDS, then out (the staging areas lie in the ring)
+  float* const F = reinterpret_cast<float*>(smem + wave * (QF_FLOATS * 4));
+  float* const RA = reinterpret_cast<float*>(smem + 4 * (QF_FLOATS * 4) + wave * 128);
+  if (use_e && g.row_alpha && lane < 32) RA[lane] = ra;
+  stage_store<0, 1>(acc, F, lane);
+  const bool diag = g.symmetric && ti == tj;
+  epilogue_quarter<F16>(g, diag, F, e_buf, RA, 0, row0, col0, lane, 0, 8, 3);
+}
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
@@ -583,12 +697,14 @@ static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
   f.reduce_tile0 = ksplit > 1 ? 0 : (f.split > 1 ? f.rounds * grid : num_tiles);
 }
 
-bool gemm_fast_eligible(const GemmArgs& a) {
+// what both tile shapes ask of a problem: whole tiles of edge `tile`, whole k stages, 16-byte
+// accesses everywhere
+static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
   if (a.f16 && a.E) return false;
   if (a.Kc < BKF || a.Kc % BKF != 0) return false;
   if (a.lda % 8 != 0 || a.ldb % 8 != 0) return false;
   if ((reinterpret_cast<uintptr_t>(a.A) & 15) || (reinterpret_cast<uintptr_t>(a.B) & 15)) return false;
-  if (a.Ma % BM != 0 || a.Nb % BN != 0) return false;           // whole tiles only: no edge masks here
+  if (a.Ma % tile != 0 || a.Nb % tile != 0) return false;       // whole tiles only: no edge masks here
   // in-tile byte offsets stay below 2^31
   if (a.lda >= (1 << 21) || a.ldb >= (1 << 21)) return false;
   if (a.C && a.c_cs != 1) return false;
@@ -596,24 +712,38 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   // 16-byte accesses of the epilogue
   if (a.C && (a.c_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C) & 15))) return false;
   if (a.C2 && (a.c2_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C2) & 15))) return false;
-  if (a.E && a.C && (a.lde % 8 != 0 || (reinterpret_cast<uintptr_t>(a.E) & 15))) return false;
-  if (a.E && a.C2 && (!a.ET || a.ldet % 8 != 0 || (reinterpret_cast<uintptr_t>(a.ET) & 15))) return false;
+  if (a.E && (a.lde % 8 != 0 || a.lde >= (1 << 21) || (reinterpret_cast<uintptr_t>(a.E) & 15))) return false;
   if (a.row_alpha && ((reinterpret_cast<uintptr_t>(a.row_alpha) & 15) || a.bs_ra % 4 != 0)) return false;
   for (int i = 0; i < a.batch && i < kMaxBatch; ++i) {
     if (a.use_c_list && (reinterpret_cast<uintptr_t>(a.c_list[i]) & 15)) return false;
     if (a.use_c2_list && (reinterpret_cast<uintptr_t>(a.c2_list[i]) & 15)) return false;
   }
-  if (a.batch > 1 && (a.bs_a % 8 || a.bs_b % 8 || a.bs_e % 8 || a.bs_et % 8 || a.bs_c % 8 || a.bs_c2 % 8)) return false;
-  // small problems: 128x128 tiles fill the chip better than few 256x256 tiles
+  if (a.batch > 1 && (a.bs_a % 8 || a.bs_b % 8 || a.bs_e % 8 || a.bs_c % 8 || a.bs_c2 % 8)) return false;
+  return true;
+}
+
+bool gemm_fast_eligible(const GemmArgs& a) {
+  if (!tiled_dma_eligible(a, BM)) return false;
+  // small problems are better off with 128x128 tiles, one per workgroup
   // (FLASHMUON_FAST_MIN_UNITS overrides the threshold, e.g. 0 to exercise this path on small inputs)
   const long long tm = a.Ma / BM, tn = a.Nb / BN;
   const long long tiles = (a.symmetric ? tm * (tm + 1) / 2 : tm * tn) * (a.batch < 1 ? 1 : a.batch);
-  static const long long min_units = [] {
-    const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS");
-    return e ? std::atoll(e) : 8192LL;
-  }();
+  long long min_units = 8192;
+  if (const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS")) min_units = std::atoll(e);
   if (tiles * (a.Kc / BKF) < min_units) return false;
   return true;
+}
+
+bool gemm_mid_eligible(const GemmArgs& a) { return tiled_dma_eligible(a, MID_T); }
+
+int launch_gemm_mid(GemmArgs a, hipStream_t stream) {
+  a.tiles_m = a.Ma / MID_T;
+  a.tiles_n = a.Nb / MID_T;
+  if (a.batch < 1) a.batch = 1;
+  a.num_tiles = (a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n) * a.batch;
+  if (a.f16) hipLaunchKernelGGL(gemm_nt_mid_kernel<true>, dim3(a.num_tiles), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL(gemm_nt_mid_kernel<false>, dim3(a.num_tiles), dim3(256), 0, stream, a);
+  return (int)hipGetLastError();
 }
 
 size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric) {

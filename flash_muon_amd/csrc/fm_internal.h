@@ -80,14 +80,17 @@ __host__ __device__ inline GemmArgs batch_view(const GemmArgs& g, int b) {
   return v;
 }
 
-// Enqueue the contraction described by `args` on `stream`, on the 256x256 stream-K path when the
-// shape, the alignment and the workspace allow it and on the general tiled path otherwise.
+// Enqueue the contraction described by `args` on `stream`: on the 256x256 path when the shape, the
+// alignment and the workspace allow it, on the 128x128 copy-fed path for smaller aligned problems,
+// and on the general tiled path otherwise.
 // Returns a hipError_t value.
 int launch_gemm_nt(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
 int launch_gemm_general(GemmArgs args, hipStream_t stream);
 bool gemm_fast_eligible(const GemmArgs& a);
 size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric);
 int launch_gemm_fast(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
+bool gemm_mid_eligible(const GemmArgs& a);
+int launch_gemm_mid(GemmArgs args, hipStream_t stream);
 
 int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
                  float* partials, hipStream_t stream);

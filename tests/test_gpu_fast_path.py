@@ -1,12 +1,8 @@
 """The 256x256 path of the GEMM-shaped kernels (rounds of whole tiles, tiles cut along k where the
 chip would otherwise idle).  It is chosen by shape (whole 256-tiles, k a multiple of 64, enough k
-stages to share out); FLASHMUON_FAST_MIN_UNITS=0 is set here, before the library is loaded, so that
-small inputs take it too and the partial-tile hand-over is exercised with few, many and uneven
-parts per tile.  Integer-valued inputs make every comparison bit-exact."""
-import os
-
-os.environ["FLASHMUON_FAST_MIN_UNITS"] = "0"
-
+stages to share out); FLASHMUON_FAST_MIN_UNITS=0 is set for every test here (the library reads it at
+each launch), so that small inputs take it too and the partial-tile hand-over is exercised with few,
+many and uneven parts per tile.  Integer-valued inputs make every comparison bit-exact."""
 import pytest
 import torch
 
@@ -15,6 +11,11 @@ from tests import gpu_util
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+
+
+@pytest.fixture(autouse=True)
+def _small_inputs_take_the_256_path(monkeypatch):
+    monkeypatch.setenv("FLASHMUON_FAST_MIN_UNITS", "0")
 
 
 def _ints(shape, seed, lo=-2, hi=2):
