@@ -638,14 +638,32 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
     }
     const unsigned char* sa = smem + (s & (MID_STAGES - 1)) * MID_STAGE;
     const unsigned char* sb = sa + MID_OPER;
+    // the 5 fragment reads of substep ks+1 ride on the 4 MFMAs of substep ks
+    bf16x8_t fa[2], fb[2][4];
+    fa[0] = *reinterpret_cast<const bf16x8_t*>(sa + ao);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) fb[0][j] = *reinterpret_cast<const bf16x8_t*>(sb + bo[j]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(sa + (ao ^ (ks << 5)));
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks < 3) {
+        fa[nxt] = *reinterpret_cast<const bf16x8_t*>(sa + (ao ^ ((ks + 1) << 5)));
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(sb + (bo[j] ^ (ks << 5)));
-        acc[0][j] = mfma_32x32x16<F16>(fa, fb, acc[0][j]);
+        for (int j = 0; j < 4; ++j) fb[nxt][j] = *reinterpret_cast<const bf16x8_t*>(sb + (bo[j] ^ ((ks + 1) << 5)));
       }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[0][j] = mfma_32x32x16<F16>(fa[cur], fb[cur][j], acc[0][j]);
+      if (ks < 3) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   wait_vmcnt<0>();
