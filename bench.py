@@ -8,8 +8,8 @@ inputs resident in HBM.  Protocol of the reference's benchmark.py:49-79: W warm-
 calls bracketed by device events.  One JSON line is printed; `value` is useful TFLOP/s
 (K*M*(M+1) flop per call), `roofline` prices the same kernel against the dense bf16 MFMA peak,
 `cpu_baseline` is torch's fp32 X @ X.T on the host cores of the same machine.  `extras` holds the
-other timings of the path: vendor GEMM X @ X.T on the same GPU, fast_newtonschulz(5) on 8192^2
-and 4096 x 16384, and Muon.step on Llama-7B shapes.
+other timings of the path: vendor GEMM X @ X.T on the same GPU, the smaller sizes of the square
+sweep, fast_newtonschulz(5) on 8192^2 and 4096 x 16384, and Muon.step on Llama-7B shapes.
 """
 import argparse
 import json
@@ -91,6 +91,17 @@ def _extras(Xd, steps, warmup, torch):
         except Exception as e:   # report, never hide
             ex["torch_xxt_%s_ms" % name] = "failed: %s" % e
     torch.backends.cuda.preferred_blas_library("default")
+    # the smaller sizes of the square sweep (seed = dim; 1024 is the CPU-sized case, seed 0)
+    from flash_muon_amd import matmul_transpose
+    for dim, seed in ((1024, 0), (2048, 2048), (4096, 4096)):
+        Xs = synthetic.gaussian_bf16(dim, dim, seed).cuda()
+        ours = _time_gpu(lambda: matmul_transpose(Xs), steps, warmup, torch)
+        ref = _time_gpu(lambda: torch.matmul(Xs, Xs.T), steps, warmup, torch)
+        ex["xxt_%d_ms" % dim] = ours
+        ex["xxt_%d_useful_tflops" % dim] = synthetic.syrk_useful_flop(dim, dim) / ours / 1e9
+        ex["torch_xxt_%d_ms" % dim] = ref
+        ex["xxt_%d_speedup_vs_torch" % dim] = ref / ours
+        del Xs
     # fast_newtonschulz(5)
     for rows, cols, rank, seed in ((8192, 8192, 16, 4), (4096, 16384, 8, 3)):
         g = torch.Generator(device="cuda").manual_seed(seed)
