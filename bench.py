@@ -45,7 +45,7 @@ def _time_gpu(fn, steps, warmup, torch):
     return start.elapsed_time(end) / steps   # ms per call
 
 
-def _cpu_baseline(X, torch):
+def _cpu_baseline(X, torch, ns=True):
     """torch fp32 X @ X.T on the host (the reference's own baseline, benchmark.py:20-21)."""
     from oracle import oracle
     M, K = X.shape
@@ -58,10 +58,24 @@ def _cpu_baseline(X, torch):
         oracle.xxt(X)
     dt = (time.perf_counter() - t0) / reps
     from flash_muon_amd import synthetic
-    return {"value": synthetic.syrk_useful_flop(M, K) / dt / 1e12, "unit": "TFLOP/s (useful)",
-            "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "torch CPU fp32 X@X.T on the full %dx%d input, 1 warm-up + %d reps, %.2f s each; "
-                      "os.cpu_count()=%d" % (M, K, reps, dt, os.cpu_count())}
+    out = {"value": synthetic.syrk_useful_flop(M, K) / dt / 1e12, "unit": "TFLOP/s (useful)",
+           "cores": torch.get_num_threads(), "kind": "port",
+           "sample": "torch CPU fp32 X@X.T on the full %dx%d input, 1 warm-up + %d reps, %.2f s each; "
+                     "os.cpu_count()=%d" % (M, K, reps, dt, os.cpu_count())}
+    if ns:
+        # the fp32 Newton-Schulz oracle on the rectangular case, once (6.2 TFLOP), and the distance of
+        # the GPU result from it on the same input
+        from flash_muon_amd import fast_newtonschulz
+        rows, cols = 4096, 16384
+        G = synthetic.gradient_like_bf16(rows, cols, 8, 3)
+        t0 = time.perf_counter()
+        ref = oracle.newtonschulz(G, 5)
+        ns_s = time.perf_counter() - t0
+        got = fast_newtonschulz(G.cuda(), 5).cpu()
+        out["ns5_4096x16384_cpu_s"] = ns_s
+        out["ns5_4096x16384_cpu_tflops"] = 5 * (4.0 * rows * rows * cols + 2.0 * rows ** 3) / ns_s / 1e12
+        out["ns5_4096x16384_gpu_vs_cpu_rel_fro"] = float(oracle.rel_fro(got, ref))
+    return out
 
 
 def _torch_ns(G, steps, torch):
@@ -102,11 +116,11 @@ def _extras(Xd, steps, warmup, torch):
         ex["torch_xxt_%d_ms" % dim] = ref
         ex["xxt_%d_speedup_vs_torch" % dim] = ref / ours
         del Xs
-    # fast_newtonschulz(5)
+    # fast_newtonschulz(5) on the gradient-like inputs of the rectangular and the square case
+    # (noise of std 1e-3 plus a rank-r spike, Frobenius-normalised; generated on the CPU from the
+    # seed so that the CPU oracle sees the same bits)
     for rows, cols, rank, seed in ((8192, 8192, 16, 4), (4096, 16384, 8, 3)):
-        g = torch.Generator(device="cuda").manual_seed(seed)
-        G = (1e-3 * torch.randn(rows, cols, generator=g, device="cuda", dtype=torch.float32))
-        G = (G / G.norm()).bfloat16()
+        G = synthetic.gradient_like_bf16(rows, cols, rank, seed).cuda()
         ms = _time_gpu(lambda: fast_newtonschulz(G, 5), 10, 3, torch)
         fl = synthetic.ns_useful_flop(rows, cols, 5)
         ex["ns5_%dx%d_ms" % (rows, cols)] = ms
@@ -182,7 +196,7 @@ def main():
                      "flop_per_launch": useful, "kernel": "gemm_nt_rounds_kernel (+ gemm_nt_reduce_kernel)"},
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = _cpu_baseline(X, torch)
+        line["cpu_baseline"] = _cpu_baseline(X, torch, ns=not args.no_extras)
     if not args.no_extras:
         ex = _extras(Xd, args.steps, args.warmup, torch)
         for k in ("torch_xxt_rocblas_ms", "torch_xxt_hipblaslt_ms"):
