@@ -1,5 +1,7 @@
 """GPU parity of Muon.step (world_size == 1) against the fp32 CPU oracle and the closed forms of
 the first and second step (flash_muon/muon.py:76-110)."""
+import copy
+
 import pytest
 import torch
 
@@ -132,6 +134,31 @@ def test_groups_state_dict_and_missing_grad():
     params[0].grad = None
     with pytest.raises(AssertionError):
         opt.step()
+
+
+def test_state_dict_round_trip_continues_identically():
+    """A second optimizer that loads the first one's state after step 1 takes the same step 2."""
+    shapes = [(128, 128), (256, 128), (128, 128)]
+    ps, gs = _make(shapes, 21)
+    a = _device_params(ps, gs)
+    opt_a = Muon(a, lr=LR, momentum=MU, rank=0, world_size=1)
+    opt_a.step()
+    b = [torch.nn.Parameter(q.detach().clone()) for q in a]
+    opt_b = Muon(b, lr=LR, momentum=MU, rank=0, world_size=1)
+    # through a deep copy, as through torch.save / torch.load: load_state_dict itself keeps the
+    # tensors it is given, and the two optimizers must not share momentum buffers
+    opt_b.load_state_dict(copy.deepcopy(opt_a.state_dict()))
+    for q, r in zip(a, b):
+        assert torch.equal(opt_a.state[q]["momentum_buffer"], opt_b.state[r]["momentum_buffer"])
+    _, gs2 = _make(shapes, 22)
+    for q, r, g in zip(a, b, gs2):
+        q.grad = g.clone().to(DEV)
+        r.grad = g.clone().to(DEV)
+    opt_a.step()
+    opt_b.step()
+    for q, r in zip(a, b):
+        assert torch.equal(q, r)
+        assert torch.equal(opt_a.state[q]["momentum_buffer"], opt_b.state[r]["momentum_buffer"])
 
 
 def test_batched_step_matches_unbatched():
