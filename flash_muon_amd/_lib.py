@@ -27,6 +27,7 @@ SIGNATURES = {
     "fm_gemm_workspace_bytes": (_sz, [_i32, _i32]),
     "fm_syrk_bf16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
     "fm_syrk_f16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
+    "fm_syrk_f32": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
     "fm_syrk_poly_bf16": (_i32, [_vp, _i64, _vp, _i64, _i32, _f32, _f32, _vp, _vp, _sz, _vp]),
     "fm_gemm_axpby_bf16": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32, _i32,
                                   _f32, _vp, _vp, _sz, _vp]),

@@ -76,32 +76,38 @@ size_t fm_gemm_workspace_bytes(int rows_out, int cols_out) {
 }
 
 static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
-                     void* ws, size_t ws_bytes, fm_stream_t stream, int f16) {
+                     void* ws, size_t ws_bytes, fm_stream_t stream, int elem) {
   if (M < 0 || K < 0) return FM_ERR_SHAPE;
   if (M == 0) return FM_OK;
   if (!X && K > 0) return FM_ERR_NULL;
   if (!Y) return FM_ERR_NULL;
   if (ldx < K) return FM_ERR_STRIDE;
   if (ldy_row == 0 || ldy_col == 0) return FM_ERR_STRIDE;
-  if (misaligned(X, 2) || misaligned(Y, 2)) return FM_ERR_ALIGN;
+  const int es = elem == kElemF32 ? 4 : 2;
+  if (misaligned(X, es) || misaligned(Y, es)) return FM_ERR_ALIGN;
   GemmArgs a = {};
   a.A = a.B = static_cast<const bf16_t*>(X); a.lda = a.ldb = ldx;
   a.E = nullptr; a.lde = 0;
   a.C = a.C2 = static_cast<bf16_t*>(Y);
   a.c_rs = a.c2_rs = ldy_row; a.c_cs = a.c2_cs = ldy_col;
   a.Ma = a.Nb = M; a.Kc = K;
-  a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1; a.f16 = f16;
+  a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1; a.elem = elem;
   return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, static_cast<hipStream_t>(stream)));
 }
 
 int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
                  void* ws, size_t ws_bytes, fm_stream_t stream) {
-  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, 0);
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, kElemBf16);
 }
 
 int fm_syrk_f16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
                 void* ws, size_t ws_bytes, fm_stream_t stream) {
-  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, 1);
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, kElemF16);
+}
+
+int fm_syrk_f32(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
+                void* ws, size_t ws_bytes, fm_stream_t stream) {
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, kElemF32);
 }
 
 int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, float b, float c,

@@ -1,14 +1,13 @@
-// bf16 (or fp16) MFMA contraction for gfx950: acc = A * B^T with both operands k-contiguous ("NT"),
-// fp32 accumulation in 32x32x16 MFMA tiles, LDS double buffering, fused epilogue and an
-// optional mirrored (transposed) second store.  X*X^T, b*A + c*A*A and a*X + P*X are all
-// instances of it (see GemmArgs).
+// MFMA contraction for gfx950, any shape, stride and alignment: acc = A * B^T with both operands
+// k-contiguous ("NT"), fp32 accumulation in 32x32 MFMA tiles (32x32x16 for bf16 and fp16 operands,
+// 32x32x2 for fp32 operands), LDS double buffering, fused epilogue and an optional mirrored
+// (transposed) second store.  X*X^T, b*A + c*A*A and a*X + P*X are all instances of it (see GemmArgs).
 #include "fm_internal.h"
 #include <cstdlib>
 
 namespace fm {
 
-constexpr int BK = 64;                 // k extent of one LDS stage: 64 bf16 = 128 bytes per row
-constexpr int ROW_BYTES = BK * 2;
+constexpr int ROW_BYTES = 128;         // one LDS row: the k extent of a stage, 64 16-bit or 32 32-bit elements
 
 // 16-byte chunk c of LDS row r lives at chunk position c ^ swz(r).  Any 8 consecutive rows get 8
 // distinct positions within a 128-byte bank group and any 16 consecutive rows get 16 distinct
@@ -32,24 +31,26 @@ __device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
   j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
 }
 
-template <int ROWS, int NT, bool ALIGNED>
+// ES: bytes per element (2 or 4).  A 16-byte chunk holds 16 / ES consecutive k.
+template <int ROWS, int NT, bool ALIGNED, int ES>
 struct TileLoader {
   static constexpr int N = ROWS * 8 / NT;   // 16-byte chunks per thread
+  static constexpr int EPC = 16 / ES;       // elements per chunk
   static_assert(ROWS * 8 % NT == 0, "tile rows must divide over the threads");
-  const bf16_t* ptr[N];   // row base + chunk offset, per chunk
-  uint32_t soff[N];       // swizzled LDS byte offset, per chunk
-  int kch[N];             // k offset of the chunk inside a stage
+  const unsigned char* ptr[N];   // row base + chunk offset, per chunk
+  uint32_t soff[N];              // swizzled LDS byte offset, per chunk
+  int kch[N];                    // k offset of the chunk inside a stage
 
-  __device__ __forceinline__ void init(const bf16_t* base, int64_t ld, int row0, int nrows, int tid) {
+  __device__ __forceinline__ void init(const void* base, int64_t ld, int row0, int nrows, int tid) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       int idx = tid + i * NT;
       int row = idx >> 3, ch = idx & 7;
       int grow = row0 + row;
       if (grow > nrows - 1) grow = nrows - 1;   // rows past the end repeat the last row; never stored
-      ptr[i] = base + (int64_t)grow * ld + ch * 8;
+      ptr[i] = static_cast<const unsigned char*>(base) + ((int64_t)grow * ld + ch * EPC) * ES;
       soff[i] = lds_off(row, ch);
-      kch[i] = ch * 8;
+      kch[i] = ch * EPC;
     }
   }
 
@@ -57,14 +58,21 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       int k = k0 + kch[i];
+      const unsigned char* src = ptr[i] + (int64_t)k0 * ES;
       if (ALIGNED) {
-        if (k < K) r[i] = *reinterpret_cast<const uint4*>(ptr[i] + k0);
+        if (k < K) r[i] = *reinterpret_cast<const uint4*>(src);
         else r[i] = make_uint4(0, 0, 0, 0);
-      } else {
+      } else if (ES == 2) {
         union { uint4 v; unsigned short h[8]; } u;
-        const unsigned short* s = reinterpret_cast<const unsigned short*>(ptr[i] + k0);
+        const unsigned short* s = reinterpret_cast<const unsigned short*>(src);
 #pragma unroll
         for (int e = 0; e < 8; ++e) u.h[e] = (k + e < K) ? s[e] : (unsigned short)0;
+        r[i] = u.v;
+      } else {
+        union { uint4 v; uint32_t w[4]; } u;
+        const uint32_t* s = reinterpret_cast<const uint32_t*>(src);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u.w[e] = (k + e < K) ? s[e] : 0u;
         r[i] = u.v;
       }
     }
@@ -76,12 +84,29 @@ struct TileLoader {
   }
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED, bool F16>
+// One 16-byte fragment pair into the accumulator: one 32x32x16 MFMA for 16-bit elements; for fp32
+// the chunk holds 4 consecutive k of this lane's k group, which are 4 steps of the 32x32x2 MFMA
+// (A and B use the same k order, and a sum does not care which order that is).
+template <int ET>
+__device__ __forceinline__ f32x16_t mfma_chunk(bf16x8_t a, bf16x8_t b, f32x16_t c) {
+  if constexpr (ET == kElemF32) {
+    const f32x4_t fa = __builtin_bit_cast(f32x4_t, a), fb = __builtin_bit_cast(f32x4_t, b);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[e], fb[e], c, 0, 0, 0);
+    return c;
+  } else {
+    return mfma_32x32x16<ET == kElemF16>(a, b, c);
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED, int ET>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArgs pb) {
   const GemmArgs p = batch_view(pb, (int)blockIdx.y);
   constexpr int NT = 64 * WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int ES = ET == kElemF32 ? 4 : 2;
+  constexpr int BK = ROW_BYTES / ES;     // elements of k per stage
   constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
   constexpr int STAGE = A_BYTES + B_BYTES;
 
@@ -101,8 +126,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
   }
   const int m0 = ti * BM, n0 = tj * BN;
 
-  TileLoader<BM, NT, ALIGNED> la;
-  TileLoader<BN, NT, ALIGNED> lb;
+  TileLoader<BM, NT, ALIGNED, ES> la;
+  TileLoader<BN, NT, ALIGNED, ES> lb;
   la.init(p.A, p.lda, m0, p.Ma, tid);
   lb.init(p.B, p.ldb, n0, p.Nb, tid);
 
@@ -132,7 +157,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
   const int khalf = lane >> 5;
 
   const int nk = (p.Kc + BK - 1) / BK;
-  uint4 ra[TileLoader<BM, NT, ALIGNED>::N], rb[TileLoader<BN, NT, ALIGNED>::N];
+  uint4 ra[TileLoader<BM, NT, ALIGNED, ES>::N], rb[TileLoader<BN, NT, ALIGNED, ES>::N];
 
   la.load(ra, 0, p.Kc);
   lb.load(rb, 0, p.Kc);
@@ -149,7 +174,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
       lb.load(rb, (kt + 1) * BK, p.Kc);
     }
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
+    for (int ks = 0; ks < 4; ++ks) {   // 8 chunks per row: chunk 2*ks + khalf belongs to this lane
       bf16x8_t fa[TM], fb[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -161,7 +186,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = mfma_32x32x16<F16>(fa[i], fb[j], acc[i][j]);
+          acc[i][j] = mfma_chunk<ET>(fa[i], fb[j], acc[i][j]);
     }
     if (more) {
       la.store(nxt, ra);
@@ -188,20 +213,25 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_nt_kernel(GemmArg
           float v = acc[i][j][r];
           if (has_e) {
             const float al = p.row_alpha ? p.alpha + p.row_alpha[row] : p.alpha;
-            v = al * elem_to_f32<F16>(__builtin_bit_cast(unsigned short, p.E[(int64_t)row * p.lde + col])) + p.beta * v;
+            v = al * elem_to_f32<false>(__builtin_bit_cast(unsigned short, p.E[(int64_t)row * p.lde + col])) + p.beta * v;
           }
           if (p.diag_out && row == col) {
             p.diag_out[row] = v;
             v = 0.0f;
           }
-          unsigned short h = f32_to_elem<F16>(v);
           // On a diagonal tile only the elements on or above the diagonal are kept, and the
           // strictly-upper ones are mirrored, so the two triangles come from the same register.
-          if (!diag || col >= row) {
-            if (C) C[(int64_t)row * p.c_rs + (int64_t)col * p.c_cs] = h;
-          }
-          if (C2 && (!p.symmetric || (diag ? col > row : true))) {
-            C2[(int64_t)col * p.c2_rs + (int64_t)row * p.c2_cs] = h;
+          const bool direct = C && (!diag || col >= row);
+          const bool mirror = C2 && (!p.symmetric || (diag ? col > row : true));
+          const int64_t o1 = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
+          const int64_t o2 = (int64_t)col * p.c2_rs + (int64_t)row * p.c2_cs;
+          if constexpr (ET == kElemF32) {
+            if (direct) reinterpret_cast<float*>(p.C)[o1] = v;
+            if (mirror) reinterpret_cast<float*>(p.C2)[o2] = v;
+          } else {
+            const unsigned short h = f32_to_elem<ET == kElemF16>(v);
+            if (direct) C[o1] = h;
+            if (mirror) C2[o2] = h;
           }
         }
       }
@@ -215,22 +245,23 @@ static int launch_cfg(GemmArgs a, bool aligned, hipStream_t stream) {
   a.tiles_n = (a.Nb + BN - 1) / BN;
   a.num_tiles = a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n;   // per matrix here
   dim3 grid((unsigned)a.num_tiles, (unsigned)a.batch), block(64 * WAVES_M * WAVES_N);
-  if (a.f16) {
-    if (aligned)
-      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true, true>), grid, block, 0, stream, a);
-    else
-      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false, true>), grid, block, 0, stream, a);
-  } else {
-    if (aligned)
-      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true, false>), grid, block, 0, stream, a);
-    else
-      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false, false>), grid, block, 0, stream, a);
-  }
+#define FM_LAUNCH_GENERAL(ET)                                                                              \
+  do {                                                                                                    \
+    if (aligned)                                                                                          \
+      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, true, ET>), grid, block, 0, stream, a);  \
+    else                                                                                                  \
+      hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, WAVES_M, WAVES_N, false, ET>), grid, block, 0, stream, a); \
+  } while (0)
+  if (a.elem == kElemF32) FM_LAUNCH_GENERAL(kElemF32);
+  else if (a.elem == kElemF16) FM_LAUNCH_GENERAL(kElemF16);
+  else FM_LAUNCH_GENERAL(kElemBf16);
+#undef FM_LAUNCH_GENERAL
   return (int)hipGetLastError();
 }
 
 int launch_gemm_general(GemmArgs a, hipStream_t stream) {
-  const bool aligned = (a.lda % 8 == 0) && (a.ldb % 8 == 0) && (a.Kc % 8 == 0) &&
+  const int epc = a.elem == kElemF32 ? 4 : 8;   // elements per 16-byte chunk
+  const bool aligned = (a.lda % epc == 0) && (a.ldb % epc == 0) && (a.Kc % epc == 0) &&
                        ((reinterpret_cast<uintptr_t>(a.A) & 15) == 0) &&
                        ((reinterpret_cast<uintptr_t>(a.B) & 15) == 0);
   // Large outputs take 256x256 tiles (8 waves, 128x64 per wave); small ones take 128x128 tiles

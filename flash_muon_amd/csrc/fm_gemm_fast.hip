@@ -718,7 +718,7 @@ static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
 // what both tile shapes ask of a problem: whole tiles of edge `tile`, whole k stages, 16-byte
 // accesses everywhere
 static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
-  if (a.f16 && a.E) return false;
+  if (a.elem == kElemF32 || (a.elem == kElemF16 && a.E)) return false;
   if (a.Kc < BKF || a.Kc % BKF != 0) return false;
   if (a.lda % 8 != 0 || a.ldb % 8 != 0) return false;
   if ((reinterpret_cast<uintptr_t>(a.A) & 15) || (reinterpret_cast<uintptr_t>(a.B) & 15)) return false;
@@ -759,7 +759,7 @@ int launch_gemm_mid(GemmArgs a, hipStream_t stream) {
   a.tiles_n = a.Nb / MID_T;
   if (a.batch < 1) a.batch = 1;
   a.num_tiles = (a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n) * a.batch;
-  if (a.f16) hipLaunchKernelGGL(gemm_nt_mid_kernel<true>, dim3(a.num_tiles), dim3(256), 0, stream, a);
+  if (a.elem == kElemF16) hipLaunchKernelGGL(gemm_nt_mid_kernel<true>, dim3(a.num_tiles), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(gemm_nt_mid_kernel<false>, dim3(a.num_tiles), dim3(256), 0, stream, a);
   return (int)hipGetLastError();
 }
@@ -785,7 +785,7 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   if (reduce_tiles > 0 && (!ws || slots > kMaxSlots || ws_bytes < (size_t)slots * PART_FLOATS * sizeof(float) ||
                            f.ksplit * f.split > kMaxParts))
     return -1;
-  if (a.f16) {
+  if (a.elem == kElemF16) {
     hipLaunchKernelGGL(gemm_nt_rounds_kernel<true>, dim3(f.grid), dim3(256), 0, stream, f);
     if (reduce_tiles > 0)
       hipLaunchKernelGGL(gemm_nt_reduce_kernel<true>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);

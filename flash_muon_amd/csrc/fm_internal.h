@@ -13,6 +13,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
 constexpr int kMaxBatch = 8;          // matrices per batched launch
+constexpr int kElemBf16 = 0, kElemF16 = 1, kElemF32 = 2;
 
 // The GEMM kernels exist for two 16-bit element types with the same memory layout; pointers are
 // typed bf16_t in both cases and F16 says what the bits mean.
@@ -39,7 +40,8 @@ template <bool F16> __device__ __forceinline__ float elem_to_f32(unsigned short 
 //     if diag_out and i == j:  diag_out[i] = v (fp32) and v = 0
 //     C [i*c_rs  + j*c_cs ] = round(v)               (if C  != nullptr)
 //     C2[j*c2_rs + i*c2_cs] = round(v)               (if C2 != nullptr; the mirrored copy)
-// A, B, E, C and C2 hold bf16, or fp16 when `f16` is set (fp16 is served without E only).
+// A, B, E, C and C2 hold bf16; without E they may hold fp16 or fp32 instead (`elem`; pointers stay
+// typed bf16_t, leading dimensions and strides stay in elements).
 // With `symmetric` set, A == B, only tiles on or above the diagonal are computed and C2 == C.
 struct GemmArgs {
   const bf16_t* A;  int64_t lda;
@@ -52,7 +54,7 @@ struct GemmArgs {
   const float* row_alpha;   // optional per-row addition to alpha
   float* diag_out;          // optional fp32 copy of the diagonal, which is then stored as zero
   int symmetric;
-  int f16;                  // element type of A, B, C, C2: 0 = bf16, 1 = fp16
+  int elem;                 // element type of A, B, C, C2: kElemBf16, kElemF16, or kElemF32 (general path only)
   // `batch` independent problems of the same shape in one launch: matrix b of an operand starts
   // b * stride elements after matrix 0 (strides of absent operands are ignored)
   int batch;

@@ -2,14 +2,14 @@
 
 Same signatures, argument checks and messages as the reference wrappers
 (flash_muon/matmul_transpose_triton.py:78-107); the Triton launch at :90-101 is replaced by
-fm_syrk_bf16 (fm_syrk_f16 for float16 tensors) from libflashmuon_hip.so.
+fm_syrk_bf16 (fm_syrk_f16 / fm_syrk_f32 for float16 / float32 tensors) from libflashmuon_hip.so.
 """
 import torch
 
 from . import _lib
 
 # the element type comes from the input, as in the reference's kernel (matmul_transpose_triton.py:63)
-_ENTRY = {torch.bfloat16: "fm_syrk_bf16", torch.float16: "fm_syrk_f16"}
+_ENTRY = {torch.bfloat16: "fm_syrk_bf16", torch.float16: "fm_syrk_f16", torch.float32: "fm_syrk_f32"}
 
 
 def matmul_transpose_assign(d_in, d_out):
@@ -27,7 +27,7 @@ def matmul_transpose_assign(d_in, d_out):
     assert d_in.size(0) == d_out.size(0) == d_out.size(1), \
         "First dimension of `d_in` must match first and second dimension of `d_out`"
     if d_in.dtype not in _ENTRY:
-        raise TypeError("matmul_transpose: bfloat16 and float16 are implemented on this device path, got %s"
+        raise TypeError("matmul_transpose: bfloat16, float16 and float32 are implemented on this device path, got %s"
                         % d_in.dtype)
     entry = _ENTRY[d_in.dtype]
 
@@ -40,7 +40,8 @@ def matmul_transpose_assign(d_in, d_out):
     ldx = d_in.stride(0) if K > 0 and M > 1 else max(K, 1)
     lib = _lib.load()
     with torch.cuda.device(d_in.device):
-        ws, ws_bytes = _lib.workspace(lib.fm_gemm_workspace_bytes(M, M), d_in.device)
+        need = 0 if d_in.dtype == torch.float32 else lib.fm_gemm_workspace_bytes(M, M)
+        ws, ws_bytes = _lib.workspace(need, d_in.device)
         st = getattr(lib, entry)(d_in.data_ptr(), ldx, d_out.data_ptr(),
                                  d_out.stride(0) if M > 1 else M, d_out.stride(1) if M > 1 else 1,
                                  M, K, ws.data_ptr() if ws is not None else None, ws_bytes,

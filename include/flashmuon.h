@@ -55,7 +55,7 @@ FM_API const char* fm_version(void);
 
 /* ---------------------------------------------------------------------------------------------
  * Scratch for the three GEMM-shaped entry points below, by the shape of their OUTPUT: (M, M) for
- * fm_syrk_bf16, fm_syrk_f16 and fm_syrk_poly_bf16, (M, K) for fm_gemm_axpby_bf16.  It holds the
+ * fm_syrk_bf16, fm_syrk_f16, fm_syrk_f32 and fm_syrk_poly_bf16, (M, K) for fm_gemm_axpby_bf16.  It holds the
  * fp32 partial tiles of output tiles whose k range is split over several workgroups.
  * The calls also run with ws == NULL (or a smaller ws) on a slower schedule that needs none.
  */
@@ -76,6 +76,12 @@ FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, in
  * to fp16, same arguments and schedule.
  */
 FM_API int fm_syrk_f16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
+                int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
+
+/* The same product for fp32 X and Y, on fp32 MFMA (32x32x2): fp32 products and accumulation, no
+ * rounding of the result.  Runs on the general tiled schedule for every shape; ws is not used.
+ */
+FM_API int fm_syrk_f32(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
                 int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------

@@ -121,7 +121,7 @@ def test_argument_contract_on_device():
     with pytest.raises(AssertionError, match="must be a CUDA tensor"):
         matmul_transpose_assign(x, torch.zeros(8, 8, dtype=torch.bfloat16))
     with pytest.raises(TypeError):
-        matmul_transpose(torch.zeros(8, 8, device=DEV))
+        matmul_transpose(torch.zeros(8, 8, dtype=torch.float64, device=DEV))
 
 
 def test_direct_c_abi_call(lib):

@@ -68,7 +68,7 @@ def test_strided_output_and_mixed_dtypes():
     with pytest.raises(AssertionError):
         matmul_transpose_assign(X, torch.empty(300, 300, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(TypeError):
-        matmul_transpose(torch.zeros(8, 8, dtype=torch.float32, device=DEV))
+        matmul_transpose(torch.zeros(8, 8, dtype=torch.int32, device=DEV))
 
 
 def test_fast_and_general_paths_agree(lib):
