@@ -85,6 +85,14 @@ static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64
   if (ldy_row == 0 || ldy_col == 0) return FM_ERR_STRIDE;
   const int es = elem == kElemF32 ? 4 : 2;
   if (misaligned(X, es) || misaligned(Y, es)) return FM_ERR_ALIGN;
+  {   // Y must not overlap X: every tile of Y is written while other tiles still read X
+    const int64_t ar = ldy_row < 0 ? -ldy_row : ldy_row, ac = ldy_col < 0 ? -ldy_col : ldy_col;
+    const int64_t back = (ldy_row < 0 ? (M - 1) * ar : 0) + (ldy_col < 0 ? (M - 1) * ac : 0);
+    Range y;
+    y.lo = reinterpret_cast<uintptr_t>(Y) - (uintptr_t)(back * es);
+    y.hi = y.lo + (uintptr_t)(((M - 1) * (ar + ac) + 1) * es);
+    if (K > 0 && overlaps(mat_range(X, M, K, ldx, es), y)) return FM_ERR_ALIAS;
+  }
   GemmArgs a = {};
   a.A = a.B = static_cast<const bf16_t*>(X); a.lda = a.ldb = ldx;
   a.E = nullptr; a.lde = 0;

@@ -65,7 +65,7 @@ FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
  * Y = X * X^T, X is M x K bf16 (row stride ldx, unit column stride), Y is M x M bf16 with
  * arbitrary strides (ldy_row, ldy_col).  Only tiles on or above the diagonal are computed; every
  * tile above it is written twice, directly and mirrored, from the same accumulators, and Y == Y^T
- * holds bit for bit.  fp32 accumulation, one round-to-nearest-even to bf16.
+ * holds bit for bit.  fp32 accumulation, one round-to-nearest-even to bf16.  Y must not overlap X.
  * Replaces mmt_kernel + its launch: flash_muon/matmul_transpose_triton.py:20-75, 90-101.
  */
 FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,

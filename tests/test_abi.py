@@ -59,6 +59,8 @@ def test_argument_errors_are_reported_before_any_launch(lib):
     assert lib.fm_syrk_bf16(X, 8, Y, 8, 1, -1, 8, None, 0, None) == 2              # shape
     assert lib.fm_syrk_bf16(ctypes.c_void_p(0x1001), 8, Y, 8, 1, 8, 8, None, 0, None) == 8   # alignment
     assert lib.fm_syrk_bf16(X, 8, Y, 8, 1, 0, 8, None, 0, None) == 0               # empty: nothing to do
+    assert lib.fm_syrk_bf16(X, 8, ctypes.c_void_p(0x1040), 8, 1, 8, 8, None, 0, None) == 5   # Y inside X
+    assert lib.fm_syrk_f32(X, 8, ctypes.c_void_p(0x1080), 1, 8, 8, 8, None, 0, None) == 5
     assert lib.fm_syrk_poly_bf16(X, 8, X, 8, 8, 1.0, 1.0, None, None, 0, None) == 5      # P aliases A
     # Xout overlapping X is rejected: every output tile reads a whole column block of X
     assert lib.fm_gemm_axpby_bf16(X, 8, Y, 8, ctypes.c_void_p(0x400000), 16, ctypes.c_void_p(0x400000), 16,
