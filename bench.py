@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the flash-muon hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--cpu-full]
 
 A step is one matmul_transpose call on the 8192 x 8192 bf16 input of the square sweep (seed 8192),
 inputs resident in HBM.  Protocol of the reference's benchmark.py:49-79: W warm-up calls, then K
@@ -45,7 +45,7 @@ def _time_gpu(fn, steps, warmup, torch):
     return start.elapsed_time(end) / steps   # ms per call
 
 
-def _cpu_baseline(X, torch, ns=True):
+def _cpu_baseline(X, torch, ns=True, full=False):
     """torch fp32 X @ X.T on the host (the reference's own baseline, benchmark.py:20-21)."""
     from oracle import oracle
     M, K = X.shape
@@ -75,6 +75,21 @@ def _cpu_baseline(X, torch, ns=True):
         out["ns5_4096x16384_cpu_s"] = ns_s
         out["ns5_4096x16384_cpu_tflops"] = 5 * (4.0 * rows * rows * cols + 2.0 * rows ** 3) / ns_s / 1e12
         out["ns5_4096x16384_gpu_vs_cpu_rel_fro"] = float(oracle.rel_fro(got, ref))
+    if full:
+        # the square Newton-Schulz case (16.5 TFLOP) and one Llama-7B layer of Muon.step (7 matrices,
+        # 21.4 TFLOP) on the CPU, once each; the step over all 32 layers is 32 times that layer
+        from flash_muon_amd import fast_newtonschulz
+        G = synthetic.gradient_like_bf16(8192, 8192, 16, 4)
+        t0 = time.perf_counter()
+        ref = oracle.newtonschulz(G, 5)
+        out["ns5_8192x8192_cpu_s"] = time.perf_counter() - t0
+        out["ns5_8192x8192_gpu_vs_cpu_rel_fro"] = float(oracle.rel_fro(fast_newtonschulz(G.cuda(), 5).cpu(), ref))
+        ps, gs = synthetic.llama7b_layer(0)
+        t0 = time.perf_counter()
+        oracle.muon_step(ps, gs, [None] * len(ps))
+        layer_s = time.perf_counter() - t0
+        out["muon_step_one_layer_cpu_s"] = layer_s
+        out["muon_step_llama7b_cpu_s_extrapolated_x32"] = 32 * layer_s
     return out
 
 
@@ -153,6 +168,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--no-extras", action="store_true", help="skip vendor GEMM, Newton-Schulz and Muon.step timings")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-full", action="store_true",
+                    help="also time the CPU oracle on Newton-Schulz 8192^2 and on one Llama-7B layer of "
+                         "Muon.step (about a minute of CPU work)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 128 MiB device-to-device copy, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -196,7 +214,7 @@ def main():
                      "flop_per_launch": useful, "kernel": "gemm_nt_rounds_kernel (+ gemm_nt_reduce_kernel)"},
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = _cpu_baseline(X, torch, ns=not args.no_extras)
+        line["cpu_baseline"] = _cpu_baseline(X, torch, ns=not args.no_extras, full=args.cpu_full)
     if not args.no_extras:
         ex = _extras(Xd, args.steps, args.warmup, torch)
         for k in ("torch_xxt_rocblas_ms", "torch_xxt_hipblaslt_ms"):
