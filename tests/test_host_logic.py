@@ -50,3 +50,15 @@ def test_synthetic_inputs_are_seeded():
     assert synthetic.ns_useful_flop(4096, 16384, 5) == synthetic.ns_useful_flop(16384, 4096, 5)
     assert abs(synthetic.ns_useful_flop(8192, 8192, 5) / 1.100e13 - 1) < 1e-3
     assert abs(synthetic.ns_useful_flop(4096, 16384, 5) / 4.467e12 - 1) < 1e-3
+
+
+def test_custom_operators_propagate_shapes_without_a_device():
+    """The torch.library registrations: fake tensors go through without touching the library."""
+    import flash_muon_amd.ops  # noqa: F401  (registers the operators)
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        x = torch.empty(48, 80, dtype=torch.bfloat16)
+        y = torch.ops.flash_muon.matmul_transpose(x)
+        assert y.shape == (48, 48) and y.dtype == torch.bfloat16
+        u = torch.ops.flash_muon.newtonschulz(torch.empty(96, 32, dtype=torch.float32), 5)
+        assert u.shape == (96, 32) and u.dtype == torch.bfloat16
