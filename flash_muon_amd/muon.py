@@ -55,16 +55,24 @@ def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
         G: The gradient or momentum matrix to be orthogonalized.
         steps: Number of Newton-Schulz iterations.
 
-    The reference asserts ndim >= 2 (muon.py:13) but its buffers and its symmetric kernel only
-    admit 2-D input (muon.py:19-20, matmul_transpose_triton.py:83); the same holds here.
+    The reference asserts ndim >= 2 (muon.py:13) and normalises over the last two dimensions
+    (muon.py:23), but its buffers and its symmetric kernel only admit 2-D input (muon.py:19-20,
+    matmul_transpose_triton.py:83).  Here leading dimensions are a batch of independent matrices,
+    orthogonalised up to 8 per launch.
     """
     assert G.ndim >= 2
-    assert G.ndim == 2, "Input `d_in` must be a 2D tensor"
     assert G.is_cuda, "Input `d_in` must be a CUDA tensor"
     if G.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         G = G.bfloat16()
     if G.numel() == 0:
         return torch.empty(G.shape, dtype=torch.bfloat16, device=G.device)
+    if G.ndim > 2:
+        flat = G.reshape(-1, G.size(-2), G.size(-1)).contiguous()
+        out = torch.empty(flat.shape, dtype=torch.bfloat16, device=G.device)
+        for i0 in range(0, flat.size(0), MAX_BATCH):
+            n = min(MAX_BATCH, flat.size(0) - i0)
+            _newtonschulz_into([flat[i0 + i] for i in range(n)], [out[i0 + i] for i in range(n)], int(steps))
+        return out.view(G.shape)
     if G.size(1) > 1 and G.stride(1) != 1 and G.stride(0) == 1 and G.stride(1) >= G.size(0):
         # a transposed view: NS(G^T) == NS(G)^T, so work on the row-major side
         return fast_newtonschulz(G.mT, steps).mT

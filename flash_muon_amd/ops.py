@@ -32,5 +32,5 @@ def newtonschulz(G: torch.Tensor, steps: int = 5) -> torch.Tensor:
 
 @newtonschulz.register_fake
 def _(G, steps=5):
-    torch._check(G.dim() == 2, lambda: "Input `d_in` must be a 2D tensor")
+    torch._check(G.dim() >= 2, lambda: "Newton-Schulz needs at least two dimensions")
     return G.new_empty(G.shape, dtype=torch.bfloat16)

@@ -139,3 +139,18 @@ def test_batched_matches_single_and_oracle(lib, rows, cols):
     assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 2)(Gs[0].data_ptr(), Gs[1].data_ptr()), 0, 2, rows, cols, cols,
                                             (ctypes.c_void_p * 2)(outs[0].data_ptr(), Gs[0].data_ptr()), cols,
                                             5, a, b, c, 1e-7, ws.data_ptr(), ws.numel(), None) == 5
+
+
+def test_leading_dimensions_are_a_batch():
+    """ndim > 2: every matrix of the leading dimensions is orthogonalised on its own (the norm of
+    muon.py:23 is over the last two dimensions), here 11 of them in chunks of 8 and 3."""
+    g = torch.Generator().manual_seed(31)
+    G = (1e-3 * torch.randn(11, 96, 160, generator=g)).bfloat16().to(DEV)
+    out = fast_newtonschulz(G, 5)
+    assert out.shape == G.shape and out.dtype == torch.bfloat16
+    for i in (0, 7, 8, 10):
+        assert torch.equal(out[i], fast_newtonschulz(G[i], 5))
+    G4 = G[:6].reshape(2, 3, 96, 160)
+    assert torch.equal(fast_newtonschulz(G4, 5), out[:6].reshape(2, 3, 96, 160))
+    tall = G[:3].mT                                  # a batch of transposed views
+    assert torch.equal(fast_newtonschulz(tall, 5), out[:3].mT)
