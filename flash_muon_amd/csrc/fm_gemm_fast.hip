@@ -21,6 +21,7 @@ constexpr int OPER_BYTES = BM * ROWB;       // one operand stage: 32 KiB
 constexpr int PART_FLOATS = BM * BN;        // one fp32 partial tile
 constexpr int kMaxParts = 64;               // parts one tile can be cut into
 constexpr int kMaxSlots = 768;              // partial-tile slots the workspace holds (192 MiB)
+constexpr int kMaxKsplit = 16;              // base parts per tile
 
 #define FM_LDS_ADDR(p) ((uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(p)))
 
@@ -292,7 +293,7 @@ struct FastArgs {
   GemmArgs g;
   float* partials;      // fp32 partial tiles
   int nk;               // k stages per tile
-  int grid;             // workgroups launched (a multiple of 8, or fewer than 8)
+  int grid;             // workgroups launched
   int ksplit;           // base parts per tile
   int rounds;           // full rounds of items
   int rem;              // items of the last, partial round
@@ -354,7 +355,10 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous block of positions
   // so that the tiles it holds at any one time are neighbours in the blocked tile order.
   int w = (int)blockIdx.x;
-  if (p.grid >= 8) w = (w & 7) * (p.grid >> 3) + (w >> 3);
+  {
+    const int chunk = p.grid >> 3;   // the workgroups past the last whole group of 8 keep their place
+    if (w < chunk * 8) w = (w & 7) * chunk + (w >> 3);
+  }
 
   const uint32_t lA0 = FM_LDS_ADDR(sA0) + wave * 1024, lB0 = FM_LDS_ADDR(sB0) + wave * 1024;
   const uint32_t lA1 = FM_LDS_ADDR(sA1) + wave * 1024, lB1 = FM_LDS_ADDR(sB1) + wave * 1024;
@@ -688,15 +692,20 @@ static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
   if (const char* e = std::getenv("FLASHMUON_GRID")) grid = std::atoi(e);   // tuning aid
   if (grid > 256) grid = 256;
   // Too few tiles for one round (M = 4096 gives 136 symmetric tiles) and a long k: cut every tile
-  // in two along k, which doubles the items at the price of one fp32 round trip per tile.
+  // along k into as many base parts as fill the chip, each at least 64 stages long so that the
+  // fp32 round trip of its partial tile stays a small part of its time.
   int ksplit = 1;
-  if (num_tiles * 5 < grid * 3 && nk >= 128) ksplit = 2;
+  if (num_tiles * 5 < grid * 3 && nk >= 128) {
+    ksplit = grid / num_tiles;
+    if (ksplit < 2) ksplit = 2;
+    if (ksplit > nk / 64) ksplit = nk / 64;
+    if (ksplit > kMaxKsplit) ksplit = kMaxKsplit;
+  }
   if (const char* e = std::getenv("FLASHMUON_KSPLIT")) ksplit = std::atoi(e);   // tuning aid
-  if (ksplit < 1 || ksplit > nk || ksplit > 4) ksplit = 1;
+  if (ksplit < 1 || ksplit > nk || ksplit > kMaxKsplit) ksplit = 1;
   if (ksplit > 1 && (int64_t)num_tiles * ksplit + grid > kMaxSlots) ksplit = 1;   // slots: items + rem * split
   const int items = num_tiles * ksplit;
   if (grid > items) grid = items;                   // rem * split never exceeds the grid below
-  if (grid >= 8) grid &= ~7;
   if (grid < 1) grid = 1;
   f.grid = grid;
   f.ksplit = ksplit;
@@ -708,6 +717,7 @@ static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
     const int base_stages = nk / ksplit;
     if (s > base_stages) s = base_stages;
     if (s > 16) s = 16;                             // bounds the partial-tile traffic
+    if (s > kMaxParts / ksplit) s = kMaxParts / ksplit;
     f.split = s < 1 ? 1 : s;
   }
   f.tail_slot0 = ksplit > 1 ? f.rounds * grid : 0;

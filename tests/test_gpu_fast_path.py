@@ -44,7 +44,7 @@ def test_syrk_fast_integer_bit_exact(lib, M, K):
     assert torch.equal(Y2, Y)
 
 
-@pytest.mark.parametrize("ksplit", [1, 2, 3, 4])
+@pytest.mark.parametrize("ksplit", [1, 2, 3, 4, 7, 16])
 @pytest.mark.parametrize("M,K", [(256, 448), (768, 1024), (1280, 8192), (4096, 1024)])
 def test_syrk_fast_forced_base_split(lib, monkeypatch, M, K, ksplit):
     """Every tile cut into `ksplit` base parts along k (the library reads the variable at each launch):
@@ -55,6 +55,47 @@ def test_syrk_fast_forced_base_split(lib, monkeypatch, M, K, ksplit):
     Y = torch.full((M, M), 7.0, dtype=torch.bfloat16, device=DEV)
     gpu_util.syrk(lib, X.to(DEV), Y)
     assert torch.equal(Y.cpu(), want)
+
+
+def test_syrk_fast_few_tiles_long_k(lib):
+    """10 tiles and 1024 k stages: every tile is cut into 16 base parts so that 160 workgroups run."""
+    X = _ints((1024, 65536), 77)
+    want = _exact(X.double() @ X.double().T)
+    Y = gpu_util.syrk(lib, X.to(DEV))
+    assert torch.equal(Y.cpu(), want)
+    assert torch.equal(Y, Y.T)
+
+
+@pytest.mark.parametrize("grid", [8, 16, 24, 40, 56])
+@pytest.mark.parametrize("M,K,ksplit", [(1280, 512, 1), (2048, 1024, 1), (2048, 448, 2), (1792, 1344, 3)])
+def test_syrk_fast_small_grids(lib, monkeypatch, M, K, ksplit, grid):
+    """Few workgroups per round (the library reads FLASHMUON_GRID at each launch): several full
+    rounds, last rounds of every fill, cut and uncut, on top of base parts."""
+    monkeypatch.setenv("FLASHMUON_GRID", str(grid))
+    monkeypatch.setenv("FLASHMUON_KSPLIT", str(ksplit))
+    X = _ints((M, K), 3 * M + K + grid)
+    want = _exact(X.double() @ X.double().T)
+    Y = torch.full((M, M), 7.0, dtype=torch.bfloat16, device=DEV)
+    gpu_util.syrk(lib, X.to(DEV), Y)
+    assert torch.equal(Y.cpu(), want)
+
+
+@pytest.mark.parametrize("grid", [8, 24, 40])
+def test_axpby_and_poly_fast_small_grids(lib, monkeypatch, grid):
+    monkeypatch.setenv("FLASHMUON_GRID", str(grid))
+    M, K = 1024, 2304
+    P = _ints((M, M), 41 + grid, -1, 1)
+    X = _ints((M, K), 43 + grid)
+    d = torch.arange(M, dtype=torch.float32) % 3 - 1
+    want = _exact((2 + d.double())[:, None] * X.double() + P.double() @ X.double())
+    Xo, XoT = gpu_util.gemm_axpby(lib, P.to(DEV), X.to(DEV), 2.0, row_alpha=d.to(DEV))
+    assert torch.equal(Xo.cpu(), want)
+    assert torch.equal(XoT.cpu(), want.T)
+    A = torch.triu(P.float()) + torch.triu(P.float(), 1).T
+    full = A.double() + 2 * (A.double() @ A.double())
+    Pp, dg = gpu_util.syrk_poly(lib, A.bfloat16().to(DEV), 1.0, 2.0, split_diag=True)
+    assert torch.equal(dg.cpu().double(), torch.diagonal(full))
+    assert torch.equal(Pp.cpu(), _exact(full - torch.diag(torch.diagonal(full))))
 
 
 @pytest.mark.parametrize("ksplit", [2, 3])
