@@ -686,21 +686,26 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
 
+// Too few tiles for one round (M = 4096 gives 136 symmetric tiles) and a long k: every tile is cut
+// along k into as many base parts as fill the chip, each at least 64 stages long so that the fp32
+// round trip of its partial tile stays a small part of its time.
+static int auto_ksplit(long long num_tiles, int nk, int grid) {
+  int ksplit = 1;
+  if (num_tiles * 5 < (long long)grid * 3 && nk >= 128) {
+    ksplit = (int)(grid / num_tiles);
+    if (ksplit < 2) ksplit = 2;
+    if (ksplit > nk / 64) ksplit = nk / 64;
+    if (ksplit > kMaxKsplit) ksplit = kMaxKsplit;
+  }
+  return ksplit;
+}
+
 // the schedule for `num_tiles` tiles of `nk` k stages
 static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
   int grid = 256;                                   // one workgroup per CU (138 KiB of LDS each)
   if (const char* e = std::getenv("FLASHMUON_GRID")) grid = std::atoi(e);   // tuning aid
   if (grid > 256) grid = 256;
-  // Too few tiles for one round (M = 4096 gives 136 symmetric tiles) and a long k: cut every tile
-  // along k into as many base parts as fill the chip, each at least 64 stages long so that the
-  // fp32 round trip of its partial tile stays a small part of its time.
-  int ksplit = 1;
-  if (num_tiles * 5 < grid * 3 && nk >= 128) {
-    ksplit = grid / num_tiles;
-    if (ksplit < 2) ksplit = 2;
-    if (ksplit > nk / 64) ksplit = nk / 64;
-    if (ksplit > kMaxKsplit) ksplit = kMaxKsplit;
-  }
+  int ksplit = auto_ksplit(num_tiles, nk, grid);
   if (const char* e = std::getenv("FLASHMUON_KSPLIT")) ksplit = std::atoi(e);   // tuning aid
   if (ksplit < 1 || ksplit > nk || ksplit > kMaxKsplit) ksplit = 1;
   if (ksplit > 1 && (int64_t)num_tiles * ksplit + grid > kMaxSlots) ksplit = 1;   // slots: items + rem * split
@@ -752,14 +757,21 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
 
 bool gemm_fast_eligible(const GemmArgs& a) {
   if (!tiled_dma_eligible(a, BM)) return false;
-  // small problems are better off with 128x128 tiles, one per workgroup
-  // (FLASHMUON_FAST_MIN_UNITS overrides the threshold, e.g. 0 to exercise this path on small inputs)
   const long long tm = a.Ma / BM, tn = a.Nb / BN;
   const long long tiles = (a.symmetric ? tm * (tm + 1) / 2 : tm * tn) * (a.batch < 1 ? 1 : a.batch);
-  long long min_units = 8192;
-  if (const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS")) min_units = std::atoll(e);
-  if (tiles * (a.Kc / BKF) < min_units) return false;
-  return true;
+  const int nk = a.Kc / BKF;
+  // FLASHMUON_FAST_MIN_UNITS replaces the choice below by a threshold on (tile, k-stage) units,
+  // e.g. 0 to exercise this path on small inputs
+  if (const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS")) return tiles * nk >= std::atoll(e);
+  // More tiles than workgroups: rounds of large tiles.  Otherwise it is one round of 256x256 tiles
+  // on some of the CUs against one or more waves of 128x128 tiles on all of them; estimate both in
+  // microseconds from the measured cost of a k stage and of a tile's epilogue on each path.
+  if (tiles > 256) return true;
+  const int ksplit = auto_ksplit(tiles, nk, 256);
+  const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
+  const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
+  const double t_small = (double)((small_tiles + 255) / 256) * (nk * 0.55 + 6.0);
+  return t_large < t_small;
 }
 
 bool gemm_mid_eligible(const GemmArgs& a) { return tiled_dma_eligible(a, MID_T); }
