@@ -42,6 +42,8 @@ SIGNATURES = {
                                             _f32, _f32, _vp, _sz, _vp]),
     "fm_momentum_nesterov": (_i32, [_vp, _vp, _i32, _i64, _f32, _f32, _i32, _vp]),
     "fm_weight_update": (_i32, [_vp, _i32, _vp, _i64, _f32, _f32, _vp]),
+    "fm_momentum_nesterov_batched": (_i32, [_vp, _vp, _i32, _i32, _i64, _f32, _f32, _i32, _vp]),
+    "fm_weight_update_batched": (_i32, [_vp, _i32, _vp, _i32, _i64, _f32, _f32, _vp]),
 }
 
 _lib = None

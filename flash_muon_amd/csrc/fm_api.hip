@@ -248,15 +248,24 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
   // tall, so the scaled cast of G is X in one case and X^T in the other.
   bf16_t* X = reinterpret_cast<bf16_t*>(w + l.x[0]);
   bf16_t* XT = reinterpret_cast<bf16_t*>(w + l.xt[0]);
-  for (int i = 0; i < batch; ++i) {
-    float* sumsq = reinterpret_cast<float*>(w + l.sumsq) + 64 * i;
-    void* partials = w + l.partials + (size_t)i * kSumsqBlocks * sizeof(float);
-    int st = fm_sumsq(G[i], dtype, rows, cols, ldg, sumsq, partials, fm_sumsq_workspace_bytes(), stream);
-    if (st) return st;
-    if (steps == 0) st = fm_scale_cast_bf16(G[i], dtype, rows, cols, ldg, sumsq, eps, out[i], ldout, nullptr, 0, stream);
-    else if (!tall) st = fm_scale_cast_bf16(G[i], dtype, rows, cols, ldg, sumsq, eps, X + i * mk, K, XT + i * mk, M, stream);
-    else            st = fm_scale_cast_bf16(G[i], dtype, rows, cols, ldg, sumsq, eps, XT + i * mk, M, X + i * mk, K, stream);
-    if (st) return st;
+  {
+    // Frobenius norms, then the scaled bf16 cast in both orientations: one launch each for the batch
+    float* sumsq = reinterpret_cast<float*>(w + l.sumsq);
+    float* partials = reinterpret_cast<float*>(w + l.partials);
+    for (int i = 0; i < batch; ++i)
+      if (misaligned(G[i], dtype_size(dtype))) return FM_ERR_ALIGN;
+    if (launch_sumsq_batched(G, batch, dtype, rows, cols, ldg, sumsq, 64, partials, hs)) return FM_ERR_LAUNCH;
+    bf16_t* d[kMaxBatch];
+    bf16_t* t[kMaxBatch];
+    for (int i = 0; i < batch; ++i) {
+      if (steps == 0) { d[i] = static_cast<bf16_t*>(out[i]); t[i] = nullptr; }
+      else if (!tall) { d[i] = X + i * mk; t[i] = XT + i * mk; }
+      else            { d[i] = XT + i * mk; t[i] = X + i * mk; }
+    }
+    const int64_t ldd = steps == 0 ? ldout : (!tall ? K : M), ldt = !tall ? M : K;
+    if (launch_scale_cast_batched(G, batch, dtype, rows, cols, ldg, sumsq, 64, eps, d, ldd,
+                                  steps == 0 ? nullptr : t, ldt, hs))
+      return FM_ERR_LAUNCH;
   }
   if (steps == 0) return FM_OK;
 
@@ -326,6 +335,47 @@ int fm_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, 
   if (overlaps(mat_range(g, 1, n, n, esz), mat_range(buf, 1, n, n, esz))) return FM_ERR_ALIAS;
   return hip_status(launch_momentum_nesterov(g, buf, dtype, n, w_buf, w_nes, nesterov,
                                              static_cast<hipStream_t>(stream)));
+}
+
+int fm_momentum_nesterov_batched(void* const* g, void* const* buf, int batch, int dtype, int64_t n,
+                                 float w_buf, float w_nes, int nesterov, fm_stream_t stream) {
+  if (bad_dtype(dtype)) return FM_ERR_DTYPE;
+  if (n < 0 || batch < 0 || batch > kMaxBatch) return FM_ERR_SHAPE;
+  if (n == 0 || batch == 0) return FM_OK;
+  if (!g || !buf) return FM_ERR_NULL;
+  const int esz = dtype_size(dtype);
+  for (int i = 0; i < batch; ++i) {
+    if (!g[i] || !buf[i]) return FM_ERR_NULL;
+    if (misaligned(g[i], esz) || misaligned(buf[i], esz)) return FM_ERR_ALIGN;
+    for (int j = 0; j < batch; ++j) {
+      if (overlaps(mat_range(g[i], 1, n, n, esz), mat_range(buf[j], 1, n, n, esz))) return FM_ERR_ALIAS;
+      if (j != i && (overlaps(mat_range(g[i], 1, n, n, esz), mat_range(g[j], 1, n, n, esz)) ||
+                     overlaps(mat_range(buf[i], 1, n, n, esz), mat_range(buf[j], 1, n, n, esz))))
+        return FM_ERR_ALIAS;
+    }
+  }
+  return hip_status(launch_momentum_nesterov_batched(g, buf, batch, dtype, n, w_buf, w_nes, nesterov,
+                                                     static_cast<hipStream_t>(stream)));
+}
+
+int fm_weight_update_batched(void* const* p, int p_dtype, const void* const* u_bf16, int batch, int64_t n,
+                             float decay_mul, float alpha, fm_stream_t stream) {
+  if (bad_dtype(p_dtype)) return FM_ERR_DTYPE;
+  if (n < 0 || batch < 0 || batch > kMaxBatch) return FM_ERR_SHAPE;
+  if (n == 0 || batch == 0) return FM_OK;
+  if (!p || !u_bf16) return FM_ERR_NULL;
+  const int esz = dtype_size(p_dtype);
+  for (int i = 0; i < batch; ++i) {
+    if (!p[i] || !u_bf16[i]) return FM_ERR_NULL;
+    if (misaligned(p[i], esz) || misaligned(u_bf16[i], 2)) return FM_ERR_ALIGN;
+    for (int j = 0; j < batch; ++j) {
+      if (overlaps(mat_range(p[i], 1, n, n, esz), mat_range(u_bf16[j], 1, n, n, 2))) return FM_ERR_ALIAS;
+      if (j != i && overlaps(mat_range(p[i], 1, n, n, esz), mat_range(p[j], 1, n, n, esz))) return FM_ERR_ALIAS;
+    }
+  }
+  return hip_status(launch_weight_update_batched(p, reinterpret_cast<const bf16_t* const*>(u_bf16), batch,
+                                                 p_dtype, n, decay_mul, alpha,
+                                                 static_cast<hipStream_t>(stream)));
 }
 
 int fm_weight_update(void* p, int p_dtype, const void* u_bf16, int64_t n, float decay_mul,

@@ -49,11 +49,15 @@ __device__ __forceinline__ float block_sum(float v, float* red /* NT/64 floats o
 }
 
 // ---- sum of squares -----------------------------------------------------------------------------
+// blockIdx.y is the matrix of a batch: its pointer comes from the list, its partial sums go to its
+// own run of gridDim.x floats
 template <int DT, bool FLAT_VEC>
-__global__ __launch_bounds__(256) void sumsq_partial_kernel(const void* Gv, int rows, int cols,
+__global__ __launch_bounds__(256) void sumsq_partial_kernel(PtrList Gl, int rows, int cols,
                                                             int64_t ldg, float* partials) {
   typedef typename Elem<DT>::raw raw;
   __shared__ float red[4];
+  const void* Gv = Gl.p[blockIdx.y];
+  partials += (size_t)blockIdx.y * gridDim.x;
   const raw* G = reinterpret_cast<const raw*>(Gv);
   const int64_t n = (int64_t)rows * cols;
   float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
@@ -83,46 +87,62 @@ __global__ __launch_bounds__(256) void sumsq_partial_kernel(const void* Gv, int 
   if (threadIdx.x == 0) partials[blockIdx.x] = s;
 }
 
-__global__ __launch_bounds__(256) void sumsq_final_kernel(const float* partials, int n, float* out) {
+// one block per matrix: its n partial sums, its own output slot
+__global__ __launch_bounds__(256) void sumsq_final_kernel(const float* partials, int n, float* out,
+                                                          int out_stride) {
   __shared__ float red[4];
+  partials += (size_t)blockIdx.x * n;
+  out += (size_t)blockIdx.x * out_stride;
   float s = 0.0f;
   for (int i = threadIdx.x; i < n; i += 256) s += partials[i];
   s = block_sum<256>(s, red);
   if (threadIdx.x == 0) out[0] = s;
 }
 
-int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
-                 float* partials, hipStream_t stream) {
+int launch_sumsq_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
+                         float* out, int out_stride, float* partials, hipStream_t stream) {
   const int64_t n = (int64_t)rows * cols;
   const int esz = dtype == 2 ? 4 : 2;
-  const bool flat = (ldg == cols) && ((reinterpret_cast<uintptr_t>(G) & 15) == 0) &&
-                    (n % (16 / esz) == 0);
-  dim3 grid(kSumsqBlocks), block(256);
-#define FM_SUMSQ(DT)                                                                              \
-  if (flat) hipLaunchKernelGGL((sumsq_partial_kernel<DT, true>), grid, block, 0, stream, G, rows, \
-                               cols, ldg, partials);                                              \
-  else hipLaunchKernelGGL((sumsq_partial_kernel<DT, false>), grid, block, 0, stream, G, rows,     \
+  bool flat = (ldg == cols) && (n % (16 / esz) == 0);
+  PtrList gl = {};
+  for (int i = 0; i < batch; ++i) {
+    gl.p[i] = const_cast<void*>(G[i]);
+    flat = flat && ((reinterpret_cast<uintptr_t>(G[i]) & 15) == 0);
+  }
+  dim3 grid(kSumsqBlocks, (unsigned)batch), block(256);
+#define FM_SUMSQ(DT)                                                                               \
+  if (flat) hipLaunchKernelGGL((sumsq_partial_kernel<DT, true>), grid, block, 0, stream, gl, rows, \
+                               cols, ldg, partials);                                               \
+  else hipLaunchKernelGGL((sumsq_partial_kernel<DT, false>), grid, block, 0, stream, gl, rows,     \
                           cols, ldg, partials);
   if (dtype == 0) { FM_SUMSQ(0) } else if (dtype == 1) { FM_SUMSQ(1) } else { FM_SUMSQ(2) }
 #undef FM_SUMSQ
-  hipLaunchKernelGGL(sumsq_final_kernel, dim3(1), dim3(256), 0, stream, (const float*)partials,
-                     kSumsqBlocks, out);
+  hipLaunchKernelGGL(sumsq_final_kernel, dim3((unsigned)batch), dim3(256), 0, stream,
+                     (const float*)partials, kSumsqBlocks, out, out_stride);
   return (int)hipGetLastError();
+}
+
+int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
+                 float* partials, hipStream_t stream) {
+  return launch_sumsq_batched(&G, 1, dtype, rows, cols, ldg, out, 0, partials, stream);
 }
 
 // ---- normalise, cast, transpose -----------------------------------------------------------------
 // One 64x64 tile of G per block: D gets the tile in place, T gets it transposed through LDS.
+// blockIdx.z is the matrix of a batch (pointers from the lists, sums of squares sumsq_stride apart).
 template <int DT>
-__global__ __launch_bounds__(256) void scale_cast_kernel(const void* Gv, int rows, int cols,
-                                                         int64_t ldg, const float* sumsq, float eps,
-                                                         unsigned short* D, int64_t ldd,
-                                                         unsigned short* T, int64_t ldt,
+__global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, int cols,
+                                                         int64_t ldg, const float* sumsq, int sumsq_stride,
+                                                         float eps, PtrList Dl, int64_t ldd,
+                                                         PtrList Tl, int64_t ldt,
                                                          int g_vec, int d_vec, int t_vec) {
   typedef typename Elem<DT>::raw raw;
   constexpr int PITCH = 66;   // u16 per LDS row: 33 dwords, so column reads spread over the banks
   __shared__ unsigned short tile[64 * PITCH];
-  const raw* G = reinterpret_cast<const raw*>(Gv);
-  const float denom = __builtin_sqrtf(sumsq[0]) + eps;
+  const raw* G = reinterpret_cast<const raw*>(Gl.p[blockIdx.z]);
+  unsigned short* D = reinterpret_cast<unsigned short*>(Dl.p[blockIdx.z]);
+  unsigned short* T = reinterpret_cast<unsigned short*>(Tl.p[blockIdx.z]);
+  const float denom = __builtin_sqrtf(sumsq[(size_t)blockIdx.z * sumsq_stride]) + eps;
   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
   const int tid = threadIdx.x;
   const int ch = tid & 7;   // 8-element chunk along the contiguous dimension
@@ -187,23 +207,33 @@ __global__ __launch_bounds__(256) void scale_cast_kernel(const void* Gv, int row
   }
 }
 
+int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
+                              const float* sumsq, int sumsq_stride, float eps, bf16_t* const* D, int64_t ldd,
+                              bf16_t* const* T, int64_t ldt, hipStream_t stream) {
+  const int esz = dtype == 2 ? 4 : 2;
+  int gv = (ldg * esz) % 16 == 0, dv = D != nullptr && ldd % 8 == 0, tv = T != nullptr && ldt % 8 == 0;
+  PtrList gl = {}, dl = {}, tl = {};
+  for (int i = 0; i < batch; ++i) {
+    gl.p[i] = const_cast<void*>(G[i]);
+    gv = gv && (reinterpret_cast<uintptr_t>(G[i]) & 15) == 0;
+    if (D) { dl.p[i] = D[i]; dv = dv && (reinterpret_cast<uintptr_t>(D[i]) & 15) == 0; }
+    if (T) { tl.p[i] = T[i]; tv = tv && (reinterpret_cast<uintptr_t>(T[i]) & 15) == 0; }
+  }
+  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch), block(256);
+#define FM_SCALE(DT) hipLaunchKernelGGL(scale_cast_kernel<DT>, grid, block, 0, stream, gl, rows, cols, ldg, \
+                                        sumsq, sumsq_stride, eps, dl, ldd, tl, ldt, gv, dv, tv)
+  if (dtype == 0) FM_SCALE(0);
+  else if (dtype == 1) FM_SCALE(1);
+  else FM_SCALE(2);
+#undef FM_SCALE
+  return (int)hipGetLastError();
+}
+
 int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
                       const float* sumsq, float eps, bf16_t* D, int64_t ldd, bf16_t* T, int64_t ldt,
                       hipStream_t stream) {
-  const int esz = dtype == 2 ? 4 : 2;
-  const int gv = ((reinterpret_cast<uintptr_t>(G) & 15) == 0) && ((ldg * esz) % 16 == 0);
-  const int dv = D && ((reinterpret_cast<uintptr_t>(D) & 15) == 0) && (ldd % 8 == 0);
-  const int tv = T && ((reinterpret_cast<uintptr_t>(T) & 15) == 0) && (ldt % 8 == 0);
-  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64)), block(256);
-  unsigned short* d = reinterpret_cast<unsigned short*>(D);
-  unsigned short* t = reinterpret_cast<unsigned short*>(T);
-  if (dtype == 0)
-    hipLaunchKernelGGL(scale_cast_kernel<0>, grid, block, 0, stream, G, rows, cols, ldg, sumsq, eps, d, ldd, t, ldt, gv, dv, tv);
-  else if (dtype == 1)
-    hipLaunchKernelGGL(scale_cast_kernel<1>, grid, block, 0, stream, G, rows, cols, ldg, sumsq, eps, d, ldd, t, ldt, gv, dv, tv);
-  else
-    hipLaunchKernelGGL(scale_cast_kernel<2>, grid, block, 0, stream, G, rows, cols, ldg, sumsq, eps, d, ldd, t, ldt, gv, dv, tv);
-  return (int)hipGetLastError();
+  return launch_scale_cast_batched(&G, 1, dtype, rows, cols, ldg, sumsq, 0, eps, D ? &D : nullptr, ldd,
+                                   T ? &T : nullptr, ldt, stream);
 }
 
 // ---- momentum + Nesterov ------------------------------------------------------------------------
@@ -220,9 +250,12 @@ __device__ __forceinline__ void momentum_one(typename Elem<DT>::raw& g, typename
   if (nesterov) g = Elem<DT>::st(lerp_torch(gf, Elem<DT>::ld(b), w_nes));
 }
 
+// blockIdx.y is the tensor of a batch
 template <int DT>
-__global__ __launch_bounds__(256) void momentum_kernel(void* gv, void* bv, int64_t n, float w_buf,
+__global__ __launch_bounds__(256) void momentum_kernel(PtrList gl, PtrList bl, int64_t n, float w_buf,
                                                        float w_nes, int nesterov, int vec) {
+  void* gv = gl.p[blockIdx.y];
+  void* bv = bl.p[blockIdx.y];
   typedef typename Elem<DT>::raw raw;
   constexpr int V = 16 / sizeof(raw);
   raw* g = reinterpret_cast<raw*>(gv);
@@ -254,23 +287,36 @@ static inline unsigned stream_grid(int64_t n_vec) {
   return (unsigned)blocks;
 }
 
-int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
-                             int nesterov, hipStream_t stream) {
-  const int vec = ((reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(buf) & 15) == 0);
+int launch_momentum_nesterov_batched(void* const* g, void* const* buf, int batch, int dtype, int64_t n,
+                                     float w_buf, float w_nes, int nesterov, hipStream_t stream) {
+  int vec = 1;
+  PtrList gl = {}, bl = {};
+  for (int i = 0; i < batch; ++i) {
+    gl.p[i] = g[i]; bl.p[i] = buf[i];
+    vec = vec && ((reinterpret_cast<uintptr_t>(g[i]) & 15) == 0) && ((reinterpret_cast<uintptr_t>(buf[i]) & 15) == 0);
+  }
   const int V = dtype == 2 ? 4 : 8;
-  dim3 grid(stream_grid(n / V + 1)), block(256);
-  if (dtype == 0) hipLaunchKernelGGL(momentum_kernel<0>, grid, block, 0, stream, g, buf, n, w_buf, w_nes, nesterov, vec);
-  else if (dtype == 1) hipLaunchKernelGGL(momentum_kernel<1>, grid, block, 0, stream, g, buf, n, w_buf, w_nes, nesterov, vec);
-  else hipLaunchKernelGGL(momentum_kernel<2>, grid, block, 0, stream, g, buf, n, w_buf, w_nes, nesterov, vec);
+  dim3 grid(stream_grid(n / V + 1), (unsigned)batch), block(256);
+  if (dtype == 0) hipLaunchKernelGGL(momentum_kernel<0>, grid, block, 0, stream, gl, bl, n, w_buf, w_nes, nesterov, vec);
+  else if (dtype == 1) hipLaunchKernelGGL(momentum_kernel<1>, grid, block, 0, stream, gl, bl, n, w_buf, w_nes, nesterov, vec);
+  else hipLaunchKernelGGL(momentum_kernel<2>, grid, block, 0, stream, gl, bl, n, w_buf, w_nes, nesterov, vec);
   return (int)hipGetLastError();
 }
 
+int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
+                             int nesterov, hipStream_t stream) {
+  return launch_momentum_nesterov_batched(&g, &buf, 1, dtype, n, w_buf, w_nes, nesterov, stream);
+}
+
 // ---- weight update ------------------------------------------------------------------------------
+// blockIdx.y is the tensor of a batch
 template <int DT>
-__global__ __launch_bounds__(256) void weight_update_kernel(void* pv, const unsigned short* u,
+__global__ __launch_bounds__(256) void weight_update_kernel(PtrList pl, PtrList ul,
                                                             int64_t n, float decay_mul, float alpha,
                                                             int vec) {
   typedef typename Elem<DT>::raw raw;
+  void* pv = pl.p[blockIdx.y];
+  const unsigned short* u = reinterpret_cast<const unsigned short*>(ul.p[blockIdx.y]);
   raw* p = reinterpret_cast<raw*>(pv);
   const int64_t stride = (int64_t)gridDim.x * 256;
   const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -300,15 +346,24 @@ __global__ __launch_bounds__(256) void weight_update_kernel(void* pv, const unsi
   }
 }
 
+int launch_weight_update_batched(void* const* p, const bf16_t* const* u, int batch, int p_dtype, int64_t n,
+                                 float decay_mul, float alpha, hipStream_t stream) {
+  int vec = 1;
+  PtrList pl = {}, ul = {};
+  for (int i = 0; i < batch; ++i) {
+    pl.p[i] = p[i]; ul.p[i] = const_cast<bf16_t*>(u[i]);
+    vec = vec && ((reinterpret_cast<uintptr_t>(p[i]) & 15) == 0) && ((reinterpret_cast<uintptr_t>(u[i]) & 15) == 0);
+  }
+  dim3 grid(stream_grid(n / 8 + 1), (unsigned)batch), block(256);
+  if (p_dtype == 0) hipLaunchKernelGGL(weight_update_kernel<0>, grid, block, 0, stream, pl, ul, n, decay_mul, alpha, vec);
+  else if (p_dtype == 1) hipLaunchKernelGGL(weight_update_kernel<1>, grid, block, 0, stream, pl, ul, n, decay_mul, alpha, vec);
+  else hipLaunchKernelGGL(weight_update_kernel<2>, grid, block, 0, stream, pl, ul, n, decay_mul, alpha, vec);
+  return (int)hipGetLastError();
+}
+
 int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float decay_mul,
                          float alpha, hipStream_t stream) {
-  const int vec = ((reinterpret_cast<uintptr_t>(p) & 15) == 0) && ((reinterpret_cast<uintptr_t>(u) & 15) == 0);
-  dim3 grid(stream_grid(n / 8 + 1)), block(256);
-  const unsigned short* uu = reinterpret_cast<const unsigned short*>(u);
-  if (p_dtype == 0) hipLaunchKernelGGL(weight_update_kernel<0>, grid, block, 0, stream, p, uu, n, decay_mul, alpha, vec);
-  else if (p_dtype == 1) hipLaunchKernelGGL(weight_update_kernel<1>, grid, block, 0, stream, p, uu, n, decay_mul, alpha, vec);
-  else hipLaunchKernelGGL(weight_update_kernel<2>, grid, block, 0, stream, p, uu, n, decay_mul, alpha, vec);
-  return (int)hipGetLastError();
+  return launch_weight_update_batched(&p, &u, 1, p_dtype, n, decay_mul, alpha, stream);
 }
 
 }  // namespace fm

@@ -92,11 +92,25 @@ int launch_gemm_fast(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t strea
 bool gemm_mid_eligible(const GemmArgs& a);
 int launch_gemm_mid(GemmArgs args, hipStream_t stream);
 
+// up to kMaxBatch device pointers, passed to a kernel by value
+struct PtrList { void* p[kMaxBatch]; };
+
+// the batched forms take HOST arrays of `batch` device pointers; matrix i reads / writes its own
+// slot of the strided arrays (out and sumsq: stride in floats; partials: kSumsqBlocks floats)
+int launch_sumsq_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
+                         float* out, int out_stride, float* partials, hipStream_t stream);
+int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
+                              const float* sumsq, int sumsq_stride, float eps, bf16_t* const* D, int64_t ldd,
+                              bf16_t* const* T, int64_t ldt, hipStream_t stream);
 int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
                  float* partials, hipStream_t stream);
 int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
                       const float* sumsq, float eps, bf16_t* D, int64_t ldd, bf16_t* T, int64_t ldt,
                       hipStream_t stream);
+int launch_momentum_nesterov_batched(void* const* g, void* const* buf, int batch, int dtype, int64_t n,
+                                     float w_buf, float w_nes, int nesterov, hipStream_t stream);
+int launch_weight_update_batched(void* const* p, const bf16_t* const* u, int batch, int p_dtype, int64_t n,
+                                 float decay_mul, float alpha, hipStream_t stream);
 int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
                              int nesterov, hipStream_t stream);
 int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float decay_mul,

@@ -139,13 +139,14 @@ class Muon(torch.optim.Optimizer):
                 g = p.grad
                 assert g is not None
                 assert p.is_cuda and g.is_cuda, "Muon parameters and gradients must be CUDA tensors"
-                buckets.setdefault((tuple(g.shape), g.dtype, g.device), []).append(p)
-            for (_, _, dev), plist in buckets.items():
+                buckets.setdefault((tuple(g.shape), g.dtype, p.dtype, g.device), []).append(p)
+            for (_, _, _, dev), plist in buckets.items():
                 staging = self._staging_rows(update.numel(), min(self.batch, len(plist)), dev)
                 for i0 in range(0, len(plist), self.batch):
                     chunk = plist[i0:i0 + self.batch]
-                    srcs = []
+                    n = len(chunk)
                     stream = _lib.stream_ptr(dev)
+                    gcs, bufs = [], []
                     for p in chunk:
                         g = p.grad
                         state = self.state[p]
@@ -154,30 +155,40 @@ class Muon(torch.optim.Optimizer):
                         buf: Tensor = state["momentum_buffer"]
                         if not buf.is_contiguous():   # e.g. a state loaded from elsewhere
                             buf = state["momentum_buffer"] = buf.contiguous()
-                        # buf.lerp_(g, 1 - mu); g.lerp_(buf, mu) in place on p.grad (muon.py:99-100)
-                        gc = g if g.is_contiguous() else g.contiguous()
-                        with torch.cuda.device(dev):
-                            st = lib.fm_momentum_nesterov(gc.data_ptr(), buf.data_ptr(), _lib.dtype_code(gc.dtype),
-                                                          gc.numel(), 1 - mu, mu, 1 if nesterov else 0, stream)
-                        _lib.check("fm_momentum_nesterov", st)
-                        if gc is not g and nesterov:
-                            g.copy_(gc)
+                        gcs.append(g if g.is_contiguous() else g.contiguous())
+                        bufs.append(buf)
+                    # buf.lerp_(g, 1 - mu); g.lerp_(buf, mu) in place on p.grad (muon.py:99-100),
+                    # one launch for the chunk
+                    with torch.cuda.device(dev):
+                        st = lib.fm_momentum_nesterov_batched(
+                            (ctypes.c_void_p * n)(*[t.data_ptr() for t in gcs]),
+                            (ctypes.c_void_p * n)(*[t.data_ptr() for t in bufs]),
+                            n, _lib.dtype_code(gcs[0].dtype), gcs[0].numel(), 1 - mu, mu,
+                            1 if nesterov else 0, stream)
+                    _lib.check("fm_momentum_nesterov_batched", st)
+                    srcs = []
+                    for p, gc, buf in zip(chunk, gcs, bufs):
+                        if gc is not p.grad and nesterov:
+                            p.grad.copy_(gc)
                         src = gc if nesterov else buf
                         if src.ndim == 4:   # conv filters (muon.py:101-102)
                             src = src.view(len(src), -1)
                         assert src.ndim == 2, "Input `d_in` must be a 2D tensor"
                         srcs.append(src)
                     # orthogonalise (muon.py:103) into rows of the staging buffer
-                    outs = [staging[i].view(srcs[i].shape) for i in range(len(chunk))]
+                    outs = [staging[i].view(srcs[i].shape) for i in range(n)]
                     _newtonschulz_into(srcs, outs, group["ns_steps"])
-                    # p *= 1 - lr*wd ; p += -lr*sqrt(max(1, rows/cols)) * update (muon.py:87-89)
-                    for i, p in enumerate(chunk):
-                        pc = p if p.is_contiguous() else p.contiguous()
-                        alpha = -lr * max(1, p.size(-2) / p.size(-1)) ** 0.5
-                        with torch.cuda.device(dev):
-                            st = lib.fm_weight_update(pc.data_ptr(), _lib.dtype_code(pc.dtype), staging[i].data_ptr(),
-                                                      pc.numel(), 1 - lr * wd, alpha, stream)
-                        _lib.check("fm_weight_update", st)
+                    # p *= 1 - lr*wd ; p += -lr*sqrt(max(1, rows/cols)) * update (muon.py:87-89),
+                    # one launch for the chunk (same shape, so the same scale)
+                    pcs = [p if p.is_contiguous() else p.contiguous() for p in chunk]
+                    alpha = -lr * max(1, chunk[0].size(-2) / chunk[0].size(-1)) ** 0.5
+                    with torch.cuda.device(dev):
+                        st = lib.fm_weight_update_batched(
+                            (ctypes.c_void_p * n)(*[t.data_ptr() for t in pcs]), _lib.dtype_code(pcs[0].dtype),
+                            (ctypes.c_void_p * n)(*[staging[i].data_ptr() for i in range(n)]),
+                            n, pcs[0].numel(), 1 - lr * wd, alpha, stream)
+                    _lib.check("fm_weight_update_batched", st)
+                    for p, pc in zip(chunk, pcs):
                         if pc is not p:
                             p.copy_(pc)
                     last = staging[len(chunk) - 1]

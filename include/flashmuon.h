@@ -183,6 +183,17 @@ FM_API int fm_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float 
 FM_API int fm_weight_update(void* p, int p_dtype, const void* u_bf16, int64_t n, float decay_mul,
                      float alpha, fm_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * The two updates above for `batch` (1..8) tensors of n elements each in one launch: g, buf, p and
+ * u_bf16 are HOST arrays of `batch` device pointers; tensor i gets exactly what the single-tensor
+ * call computes.  No tensor may overlap another.  For the loop over same-shape parameters:
+ * flash_muon/muon.py:90-100 and 86-89.
+ */
+FM_API int fm_momentum_nesterov_batched(void* const* g, void* const* buf, int batch, int dtype, int64_t n,
+                                 float w_buf, float w_nes, int nesterov, fm_stream_t stream);
+FM_API int fm_weight_update_batched(void* const* p, int p_dtype, const void* const* u_bf16, int batch,
+                             int64_t n, float decay_mul, float alpha, fm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
