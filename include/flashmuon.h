@@ -146,7 +146,7 @@ FM_API int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int6
 FM_API size_t fm_newtonschulz_workspace_bytes(int rows, int cols);
 
 /* ---------------------------------------------------------------------------------------------
- * The same for `batch` (1..8) matrices of one shape and dtype, with every GEMM-shaped stage run
+ * The same for `batch` (1..16) matrices of one shape and dtype, with every GEMM-shaped stage run
  * as ONE launch over the whole batch, so that shapes whose tile count does not fill the chip
  * (M = 4096 gives 136 tiles for 256 CUs) are packed together.  G and out are HOST arrays of
  * `batch` device pointers; all inputs share ldg and all outputs ldout.  No out[i] may overlap
@@ -184,7 +184,7 @@ FM_API int fm_weight_update(void* p, int p_dtype, const void* u_bf16, int64_t n,
                      float alpha, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
- * The two updates above for `batch` (1..8) tensors of n elements each in one launch: g, buf, p and
+ * The two updates above for `batch` (1..16) tensors of n elements each in one launch: g, buf, p and
  * u_bf16 are HOST arrays of `batch` device pointers; tensor i gets exactly what the single-tensor
  * call computes.  No tensor may overlap another.  For the loop over same-shape parameters:
  * flash_muon/muon.py:90-100 and 86-89.
