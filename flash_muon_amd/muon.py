@@ -114,15 +114,54 @@ class Muon(torch.optim.Optimizer):
         defaults = dict(lr=lr, weight_decay=weight_decay, momentum=momentum, nesterov=nesterov, ns_steps=ns_steps)
         params = [*params]
         param_groups = []
-        # one group per distinct numel, each with a [world_size, numel] bf16 update buffer
-        # (flash_muon/muon.py:68-72); sorted so that the group order does not depend on hashing
-        for size in sorted({p.numel() for p in params}):
+        # One group per distinct numel, each with a [world_size, numel] bf16 update buffer, in the
+        # iteration order of the same set expression as flash_muon/muon.py:68-72, so that groups
+        # (and with them the entries of a state_dict) come out in the reference's order.  The
+        # buffer lives where the parameters live (the reference writes "cuda", muon.py:69).
+        for size in {p.numel() for p in params}:
             members = [p for p in params if p.numel() == size]
-            b = torch.empty(world_size, size, dtype=torch.bfloat16, device=members[0].device if members[0].is_cuda else "cuda")
+            b = torch.empty(world_size, size, dtype=torch.bfloat16, device=members[0].device)
             group = dict(params=members, update_buffer=b,
                          update_buffer_views=[b[i] for i in range(world_size)])
             param_groups.append(group)
         super().__init__(param_groups, defaults)
+
+    def load_state_dict(self, state_dict):
+        """torch pairs saved and live groups by position; a checkpoint whose groups were built in
+        another order (another interpreter's set order, or a sorted one) is first put into this
+        optimizer's order by the numel of each group's update buffer, the key the groups are made
+        from (flash_muon/muon.py:68-71).  The buffers themselves are scratch: whatever their saved
+        world size or device, each group keeps a [1, numel] bf16 buffer next to its parameters."""
+        saved = state_dict["param_groups"]
+        own = [g["update_buffer"].size(-1) for g in self.param_groups]
+        theirs = [g["update_buffer"].size(-1) if torch.is_tensor(g.get("update_buffer")) else None for g in saved]
+        if theirs != own and None not in theirs and sorted(theirs) == sorted(own):
+            order = [theirs.index(n) for n in own]
+            # parameter ids are positions in the saved order: renumber them for the new order
+            remap, nxt = {}, 0
+            groups = []
+            for i in order:
+                g = dict(saved[i])
+                ids = []
+                for pid in g["params"]:
+                    remap[pid] = nxt
+                    ids.append(nxt)
+                    nxt += 1
+                g["params"] = ids
+                groups.append(g)
+            state_dict = {"state": {remap.get(k, k): v for k, v in state_dict["state"].items()},
+                          "param_groups": groups}
+        super().load_state_dict(state_dict)
+        for group in self.param_groups:
+            dev = group["params"][0].device
+            n = group["params"][0].numel()
+            b = group.get("update_buffer")
+            if not (torch.is_tensor(b) and b.shape == (1, n) and b.dtype == torch.bfloat16 and b.device == dev):
+                nb = torch.zeros(1, n, dtype=torch.bfloat16, device=dev)
+                if torch.is_tensor(b) and b.ndim == 2 and b.size(1) == n:
+                    nb[0].copy_(b[0])
+                group["update_buffer"] = nb
+            group["update_buffer_views"] = [group["update_buffer"][0]]
 
     @torch.no_grad()
     def step(self):
@@ -153,6 +192,11 @@ class Muon(torch.optim.Optimizer):
                         if "momentum_buffer" not in state:
                             state["momentum_buffer"] = torch.zeros_like(g, memory_format=torch.contiguous_format)
                         buf: Tensor = state["momentum_buffer"]
+                        # the kernel reads both through one dtype code and one element count
+                        assert buf.shape == g.shape and buf.device == g.device, \
+                            "momentum_buffer must match the gradient in shape and device"
+                        if buf.dtype != g.dtype:   # load_state_dict casts state to the parameter's dtype
+                            buf = state["momentum_buffer"] = buf.to(g.dtype)
                         if not buf.is_contiguous():   # e.g. a state loaded from elsewhere
                             buf = state["momentum_buffer"] = buf.contiguous()
                         gcs.append(g if g.is_contiguous() else g.contiguous())
@@ -191,9 +235,10 @@ class Muon(torch.optim.Optimizer):
                     for p, pc in zip(chunk, pcs):
                         if pc is not p:
                             p.copy_(pc)
-                    last = staging[len(chunk) - 1]
-                # the group's update buffer ends up holding the last update, as in muon.py:108
-                update.copy_(last)
+                    if chunk[-1] is group["params"][-1]:
+                        # the group's update buffer ends up holding the update of its last
+                        # parameter, as after the last gather of muon.py:108
+                        update.copy_(staging[len(chunk) - 1])
 
     def _staging_rows(self, numel, rows, device):
         """[rows, numel] bf16 scratch the batched orthogonalisation writes its updates to."""

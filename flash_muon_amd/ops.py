@@ -27,7 +27,9 @@ def _(x):
 
 @torch.library.custom_op("flash_muon::newtonschulz", mutates_args=())
 def newtonschulz(G: torch.Tensor, steps: int = 5) -> torch.Tensor:
-    return _fast_newtonschulz(G, steps)
+    # fast_newtonschulz answers a transposed view with a transposed view; an operator's output
+    # strides have to be what its fake kernel says, so the operator always returns contiguous
+    return _fast_newtonschulz(G, steps).contiguous()
 
 
 @newtonschulz.register_fake

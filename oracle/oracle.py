@@ -55,7 +55,8 @@ def ns_prepare(G, dtype=torch.float32):
     tall = G.size(-2) > G.size(-1)
     if tall:
         X = X.mT
-    X = X / (X.norm() + NS_EPS)
+    # the norm is taken over the last two dimensions (muon.py:23): leading ones are a batch
+    X = X / (X.norm(dim=(-2, -1), keepdim=True) + NS_EPS)
     return X.contiguous(), tall
 
 
@@ -71,7 +72,8 @@ def newtonschulz(G, steps=5, dtype=torch.float32, trace=False):
     """fast_newtonschulz computed without intermediate bf16 roundings (muon.py:6-33).
 
     Returns the result in `dtype` with G's shape; with trace=True also the list of iterates in the
-    wide orientation (X_0 after normalisation, then one per step).
+    wide orientation (X_0 after normalisation, then one per step).  Leading dimensions of G are a
+    batch of independent matrices, each normalised by its own norm (muon.py:13, 23).
     """
     X, tall = ns_prepare(G, dtype)
     states = [X]

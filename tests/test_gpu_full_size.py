@@ -1,10 +1,12 @@
 """The benchmark configurations at their full sizes: Newton-Schulz on 4096 x 16384 and 8192 x 8192
 and one Llama-7B layer of Muon.step, against the fp32 CPU oracle (a few TFLOP each on the host, so
 these are the slowest tests), plus properties that need no CPU product."""
+import ctypes
+
 import pytest
 import torch
 
-from flash_muon_amd import Muon, fast_newtonschulz, synthetic
+from flash_muon_amd import Muon, _lib, fast_newtonschulz, synthetic
 from oracle import oracle
 
 pytestmark = pytest.mark.gpu
@@ -40,23 +42,85 @@ def test_square_newtonschulz_8192():
     assert err1 < 1e-2
 
 
+def _applied_update(p_before, p_after, lr, wd):
+    """The update Muon.step applied, recovered from an fp32 parameter:
+    p' = p (1 - lr wd) - lr sqrt(max(1, rows/cols)) u   (muon.py:87-89)."""
+    scale = max(1, p_before.size(0) / p_before.size(1)) ** 0.5
+    return (p_before.double() * (1 - lr * wd) - p_after.double()) / (lr * scale)
+
+
 def test_muon_step_one_llama7b_layer():
+    """One layer of the Llama-7B configuration (4 x 4096^2, 2 x 11008x4096, 1 x 4096x11008), bf16
+    parameters and gradients, against the oracle: state, gradient, parameter, and the update itself
+    as step() applied it.  The update is read back from a second optimizer over fp32 copies of the
+    same parameters (same gradients, same batches of 4 + 2 + 1 matrices through the same kernels):
+    an fp32 parameter keeps the update to 1e-5 of its size, a bf16 parameter rounds it away."""
+    lr, wd = 0.02, 0.01
     ps, gs = synthetic.llama7b_layer(0)
-    params = []
+    params, params32 = [], []
     for p, g in zip(ps, gs):
         q = torch.nn.Parameter(p.clone().to(DEV))
         q.grad = g.clone().to(DEV)
         params.append(q)
-    opt = Muon(params, lr=0.02, momentum=0.95, nesterov=True, rank=0, world_size=1)
+        q32 = torch.nn.Parameter(p.float().to(DEV))
+        q32.grad = g.clone().to(DEV)
+        params32.append(q32)
+    opt = Muon(params, lr=lr, momentum=0.95, nesterov=True, rank=0, world_size=1)
+    opt32 = Muon(params32, lr=lr, momentum=0.95, nesterov=True, rank=0, world_size=1)
     opt.step()
-    ref_p, ref_g, ref_b, ref_u = oracle.muon_step(ps, gs, [None] * len(ps), 0.02, 0.01, 0.95, True, 5)
-    for q, p0, rp, rg, rb, ru in zip(params, ps, ref_p, ref_g, ref_b, ref_u):
+    opt32.step()
+    ref_p, ref_g, ref_b, ref_u = oracle.muon_step(ps, gs, [None] * len(ps), lr, wd, 0.95, True, 5)
+    for q, q32, p0, rp, rg, rb, ru in zip(params, params32, ps, ref_p, ref_g, ref_b, ref_u):
         assert oracle.rel_fro(opt.state[q]["momentum_buffer"], rb) < 4e-3
         assert oracle.rel_fro(q.grad, rg) < 4e-3
         assert oracle.rel_fro(q.data, rp) < 3e-3
-        # the update itself, recovered from the parameter change in fp32 terms
-        scale = max(1, p0.size(0) / p0.size(1)) ** 0.5
-        upd = fast_newtonschulz(q.grad, 5).float().cpu()
+        assert torch.equal(q32.grad, q.grad)
+        upd = _applied_update(p0.float(), q32.data.cpu(), lr, wd)
+        assert bool(torch.isfinite(upd).all())
         err = oracle.rel_fro(upd, ru)
-        print("update %s rel_fro %.3e" % (tuple(p0.shape), err), flush=True)
+        print("applied update %s rel_fro %.3e" % (tuple(p0.shape), err), flush=True)
         assert err < 1e-2
+        # the bf16 parameter moved by the same update, up to its own rounding (2^-9 of |p| ~ 0.02)
+        moved = (p0.double() * (1 - lr * wd) - q.data.cpu().double())
+        scale = max(1, p0.size(0) / p0.size(1)) ** 0.5
+        assert oracle.rel_fro(moved, lr * scale * ru.double()) < 0.2
+    # the group buffers end up holding the last update of their group (muon.py:108)
+    for group in opt32.param_groups:
+        last = group["params"][-1]
+        idx = [i for i, q in enumerate(params32) if q is last][0]
+        got = group["update_buffer"][0].view(ref_u[idx].shape)
+        assert oracle.rel_fro(got, ref_u[idx]) < 1e-2
+
+
+def _batched_ns(lib, Gs, steps=5):
+    rows, cols = Gs[0].shape
+    n = len(Gs)
+    outs = [torch.empty(rows, cols, dtype=torch.bfloat16, device=DEV) for _ in Gs]
+    a, b, c = oracle.NS_COEFFS
+    ws = torch.empty(lib.fm_newtonschulz_batched_workspace_bytes(n, rows, cols), dtype=torch.uint8, device=DEV)
+    st = lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * n)(*[g.data_ptr() for g in Gs]), 0, n, rows, cols, cols,
+                                          (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs]), cols, steps, a, b, c,
+                                          oracle.NS_EPS, ws.data_ptr(), ws.numel(), _lib.stream_ptr(Gs[0].device))
+    _lib.check("fm_newtonschulz_batched_bf16", st)
+    torch.cuda.synchronize()
+    return outs
+
+
+@pytest.mark.parametrize("rows,cols,checked", [(4096, 4096, (0, 11)), (4096, 11008, (5, 15)), (11008, 4096, (2,))])
+def test_sixteen_per_launch_schedule(lib, rows, cols, checked):
+    """fm_newtonschulz_batched_bf16 with sixteen Llama-7B-sized matrices per launch, the schedule
+    Muon.step and bench.py run: the members in `checked` against the fp32 CPU oracle, every member
+    for finite values and against the single-matrix call (which differs only in which tiles are
+    summed from parts, i.e. in fp32 summation order)."""
+    n = 16
+    Gs = [synthetic.gradient_like_bf16(rows, cols, 8, 700 + i) for i in range(n)]
+    dGs = [G.to(DEV) for G in Gs]
+    outs = _batched_ns(lib, dGs)
+    for i in checked:
+        err = oracle.rel_fro(outs[i], oracle.newtonschulz(Gs[i], 5))
+        print("batch of 16, %dx%d, member %d: rel_fro %.3e" % (rows, cols, i, err), flush=True)
+        assert err < 1e-2
+    for i in range(n):
+        assert bool(torch.isfinite(outs[i]).all())
+        single = fast_newtonschulz(dGs[i], 5)
+        assert oracle.rel_fro(outs[i], single.float()) < 4e-3

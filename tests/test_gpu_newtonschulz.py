@@ -148,6 +148,18 @@ def test_leading_dimensions_are_a_batch():
     G = (1e-3 * torch.randn(19, 96, 160, generator=g)).bfloat16().to(DEV)
     out = fast_newtonschulz(G, 5)
     assert out.shape == G.shape and out.dtype == torch.bfloat16
+    # against the CPU oracle on the whole batch (per-matrix norms, muon.py:23), every member
+    Gc = G.cpu().clone()
+    Gc[3] *= 64.0                                     # norms that differ between members
+    ref = oracle.newtonschulz(Gc, 5)
+    got = fast_newtonschulz(Gc.to(DEV), 5)
+    for i in range(G.size(0)):
+        err = oracle.rel_fro(got[i], ref[i])
+        assert err < _tol(96, 160), "member %d: %g" % (i, err)
+    tall_ref = oracle.newtonschulz(Gc[:4].mT.contiguous(), 5)
+    tall_got = fast_newtonschulz(Gc[:4].mT.contiguous().to(DEV), 5)
+    assert tall_got.shape == (4, 160, 96)
+    assert oracle.rel_fro(tall_got, tall_ref) < _tol(96, 160)
     for i in (0, 7, 15, 16, 18):
         assert torch.equal(out[i], fast_newtonschulz(G[i], 5))
     G4 = G[:6].reshape(2, 3, 96, 160)

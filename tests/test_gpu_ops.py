@@ -4,7 +4,7 @@ import pytest
 import torch
 
 import flash_muon_amd.ops  # noqa: F401  (registers the operators)
-from flash_muon_amd import fast_newtonschulz, matmul_transpose
+from flash_muon_amd import fast_newtonschulz, matmul_transpose, synthetic
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -28,3 +28,16 @@ def test_captured_graph_holds_the_operators():
     want = f(x, G)
     got = torch.compile(f, backend="aot_eager", fullgraph=True)(x, G)
     assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+def test_newtonschulz_operator_strides_match_its_fake_kernel():
+    """A transposed view in: the plain function answers with a transposed view, the operator with a
+    contiguous tensor, which is what its fake kernel promises to torch.compile."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    G = synthetic.gradient_like_bf16(96, 160, 4, 61).to(DEV)
+    real = torch.ops.flash_muon.newtonschulz(G.mT, 5)
+    assert real.shape == (160, 96) and real.is_contiguous()
+    assert torch.equal(real, fast_newtonschulz(G.mT, 5))
+    with FakeTensorMode():
+        fake = torch.ops.flash_muon.newtonschulz(torch.empty(96, 160, dtype=torch.bfloat16).mT, 5)
+    assert fake.shape == real.shape and fake.stride() == real.stride()

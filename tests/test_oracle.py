@@ -101,6 +101,80 @@ def test_ns_step_trace_consistent():
     assert torch.equal(out, st[3])
 
 
+def test_rel_fro_known_values():
+    """The parity metric itself: known non-zero answers, so that a metric that returned 0 (or the
+    wrong ratio) could not pass the floating-point tests silently."""
+    g = torch.Generator().manual_seed(2)
+    R = torch.randn(37, 53, generator=g, dtype=torch.float64)
+    assert oracle.rel_fro(R, R) == 0.0
+    assert abs(oracle.rel_fro(1.01 * R, R) - 0.01) < 1e-12
+    assert abs(oracle.rel_fro(torch.zeros_like(R), R) - 1.0) < 1e-15
+    assert abs(oracle.rel_fro(-R, R) - 2.0) < 1e-15
+    E = torch.zeros(4, 4, dtype=torch.float64)
+    E[1, 2] = 0.5                                   # ||E||_F = 0.5, ||I_4||_F = 2
+    assert abs(oracle.rel_fro(torch.eye(4, dtype=torch.float64) + E, torch.eye(4, dtype=torch.float64)) - 0.25) < 1e-15
+    # it is relative to the SECOND argument: ||R - 3R|| / ||3R|| = 2/3, not 2
+    assert abs(oracle.rel_fro(R, 3 * R) - 2.0 / 3.0) < 1e-12
+    # bf16 inputs are compared by value (one rounding of N(0,1) data is about 2^-9 / sqrt(3) relative)
+    assert 1.5e-3 < oracle.rel_fro(R.bfloat16(), R) < 3e-3
+
+
+def test_newtonschulz_leading_dimensions_are_a_batch():
+    """muon.py:13 admits ndim >= 2 and muon.py:23 normalises over the last two dimensions: every
+    matrix of a batch goes through the iteration on its own, with its own norm."""
+    g = torch.Generator().manual_seed(17)
+    G = torch.randn(3, 2, 24, 40, generator=g, dtype=torch.float64)
+    G[1] *= 1e3                                      # very different norms must not leak between matrices
+    G[2, 1] *= 1e-4
+    got = oracle.newtonschulz(G, 5, torch.float64)
+    assert got.shape == G.shape
+    for i in range(3):
+        for j in range(2):
+            U, S, Vh = torch.linalg.svd(G[i, j].bfloat16().double(), full_matrices=False)
+            s = S / (S.norm() + oracle.NS_EPS)
+            a, b, c = oracle.NS_COEFFS
+            for _ in range(5):
+                s = a * s + b * s ** 3 + c * s ** 5
+            want = U @ torch.diag(s) @ Vh
+            assert oracle.rel_fro(got[i, j], want) < 1e-9
+    # tall matrices in a batch: transposed, iterated, transposed back
+    T = G.mT.contiguous()
+    assert oracle.rel_fro(oracle.newtonschulz(T, 5, torch.float64), got.mT) < 1e-12
+    e = oracle.newtonschulz_eager_bf16(G, 5)
+    assert e.shape == G.shape and e.dtype == torch.bfloat16
+
+
+def _bf(x):
+    """Round a python float / fp32 value to bf16 and back (one torch rounding)."""
+    return float(torch.tensor(x, dtype=torch.float32).bfloat16().float())
+
+
+def test_eager_bf16_scalar_recurrence_on_a_diagonal_input():
+    """newtonschulz_eager_bf16 on diag(sigma) is a scalar recurrence per singular value in which
+    every torch op of muon.py:23-29 rounds to bf16: written out here op by op (norm, divide, A, A^2,
+    b*A, c*A^2, their sum, a*X, B@X, their sum), it has to reproduce the matrix code bit for bit.
+    A transposed operand, a dropped term or a missing rounding in the matrix code breaks it."""
+    a, b, c = oracle.NS_COEFFS
+    sig = [1.0, 0.5, 0.11, 0.013]
+    G = torch.diag(torch.tensor(sig, dtype=torch.float32))
+    got = torch.diagonal(oracle.newtonschulz_eager_bf16(G, 5)).float().tolist()
+    xs = [_bf(v) for v in sig]
+    norm = _bf(math.sqrt(sum(v * v for v in xs)))           # X.norm() comes back as a bf16 scalar
+    den = _bf(norm + oracle.NS_EPS)
+    xs = [_bf(v / den) for v in xs]
+    for _ in range(5):
+        nxt = []
+        for x in xs:
+            A = _bf(x * x)
+            A2 = _bf(A * A)
+            B = _bf(_bf(b * A) + _bf(c * A2))
+            nxt.append(_bf(_bf(a * x) + _bf(B * x)))
+        xs = nxt
+    assert got == xs
+    off = oracle.newtonschulz_eager_bf16(G, 5).float() - torch.diag(torch.tensor(got))
+    assert float(off.abs().max()) == 0.0
+
+
 def test_eager_bf16_close_to_fp32():
     g = torch.Generator().manual_seed(11)
     G = torch.randn(64, 96, generator=g)
