@@ -12,7 +12,10 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libflashmuo
 
 # fm_status values (include/flashmuon.h)
 FM_OK = 0
+FM_ERR_STRIDE = 3
 FM_ERR_ALIAS = 5
+# fm_knob values
+FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID = 0, 1, 2, 3
 FM_BF16, FM_F16, FM_F32 = 0, 1, 2
 
 _DTYPE_CODE = {torch.bfloat16: FM_BF16, torch.float16: FM_F16, torch.float32: FM_F32}
@@ -24,6 +27,7 @@ _vp, _i64, _i32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, cty
 SIGNATURES = {
     "fm_status_string": (ctypes.c_char_p, [_i32]),
     "fm_version": (ctypes.c_char_p, []),
+    "fm_set_knob": (_i32, [_i32, ctypes.c_longlong]),
     "fm_gemm_workspace_bytes": (_sz, [_i32, _i32]),
     "fm_syrk_bf16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
     "fm_syrk_f16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
@@ -95,3 +99,19 @@ def workspace(nbytes, device):
         return None, 0
     ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
     return ws, nbytes
+
+
+_gemm_ws = {}
+
+
+def gemm_workspace(nbytes, device):
+    """The partial-tile scratch of the single GEMM-shaped calls (at most 192 MiB), kept per device
+    and stream: calls on one stream are ordered, so they can share it, and nothing is allocated
+    per call."""
+    if nbytes == 0:
+        return None, 0
+    key = (torch.device(device).index, stream_ptr(device))
+    ws = _gemm_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = _gemm_ws[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws, ws.numel()

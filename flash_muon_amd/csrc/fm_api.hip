@@ -21,7 +21,7 @@ inline bool overlaps(Range a, Range b) { return a.lo < b.hi && b.lo < a.hi; }
 inline bool misaligned(const void* p, int esz) { return (reinterpret_cast<uintptr_t>(p) % esz) != 0; }
 inline int dtype_size(int dt) { return dt == FM_F32 ? 4 : 2; }
 inline bool bad_dtype(int dt) { return dt != FM_BF16 && dt != FM_F16 && dt != FM_F32; }
-inline int hip_status(int hip_err) { return hip_err == 0 ? FM_OK : FM_ERR_LAUNCH; }
+inline int hip_status(int rc) { return rc == 0 ? FM_OK : (rc == kErrWorkspace ? FM_ERR_WORKSPACE : FM_ERR_LAUNCH); }
 // a workspace is only used when it is 256-byte aligned; otherwise the call runs without one
 inline void* usable_ws(void* ws) { return (reinterpret_cast<uintptr_t>(ws) % 256 == 0) ? ws : nullptr; }
 
@@ -44,7 +44,9 @@ NsLayout ns_layout(int batch, int rows, int cols) {
   for (int i = 0; i < 2; ++i) { l.x[i] = take(B * M * K * 2); l.xt[i] = take(B * M * K * 2); }
   l.a = take(B * M * M * 2);
   l.p = take(B * M * M * 2);
-  l.gemm = take(fm_gemm_workspace_bytes((int)M, (int)K));
+  // partial tiles of the three products of a step: two M x M (symmetric) and one M x K, `batch` each
+  const size_t g1 = gemm_fast_workspace_bytes((int)M, (int)M, batch), g2 = gemm_fast_workspace_bytes((int)M, (int)K, batch);
+  l.gemm = take(g1 > g2 ? g1 : g2);
   l.total = off;
   return l;
 }
@@ -72,8 +74,10 @@ const char* fm_version(void) { return "0.1.0"; }
 
 size_t fm_gemm_workspace_bytes(int rows_out, int cols_out) {
   if (rows_out <= 0 || cols_out <= 0) return 0;
-  return gemm_fast_workspace_bytes(rows_out, cols_out, false);
+  return gemm_fast_workspace_bytes(rows_out, cols_out, 1);
 }
+
+int fm_set_knob(int which, long long value) { return set_knob(which, value) == 0 ? FM_OK : FM_ERR_SHAPE; }
 
 static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
                      void* ws, size_t ws_bytes, fm_stream_t stream, int elem) {
@@ -83,6 +87,13 @@ static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64
   if (!Y) return FM_ERR_NULL;
   if (ldx < K) return FM_ERR_STRIDE;
   if (ldy_row == 0 || ldy_col == 0) return FM_ERR_STRIDE;
+  if (M > 1) {
+    // distinct (i, j) must not share an address: the larger stride has to step over a whole line
+    // of the smaller one (true of every dense or padded row- or column-major layout)
+    const int64_t ar = ldy_row < 0 ? -ldy_row : ldy_row, ac = ldy_col < 0 ? -ldy_col : ldy_col;
+    const int64_t lo = ar < ac ? ar : ac, hi = ar < ac ? ac : ar;
+    if (hi < (int64_t)M * lo) return FM_ERR_STRIDE;
+  }
   const int es = elem == kElemF32 ? 4 : 2;
   if (misaligned(X, es) || misaligned(Y, es)) return FM_ERR_ALIGN;
   {   // Y must not overlap X: every tile of Y is written while other tiles still read X
@@ -235,6 +246,15 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
   const NsLayout l = ns_layout(batch, rows, cols);
   if (!ws || ws_bytes < l.total) return FM_ERR_WORKSPACE;
   if (reinterpret_cast<uintptr_t>(ws) % 256 != 0) return FM_ERR_ALIGN;
+  {
+    Range w;
+    w.lo = reinterpret_cast<uintptr_t>(ws);
+    w.hi = w.lo + l.total;
+    for (int i = 0; i < batch; ++i)
+      if (overlaps(mat_range(G[i], rows, cols, ldg, dtype_size(dtype)), w) ||
+          overlaps(mat_range(out[i], rows, cols, ldout, 2), w))
+        return FM_ERR_ALIAS;
+  }
 
   unsigned char* w = static_cast<unsigned char*>(ws);
   void* gws = w + l.gemm;

@@ -3,32 +3,15 @@
 // 32x32x2 for fp32 operands), LDS double buffering, fused epilogue and an optional mirrored
 // (transposed) second store.  X*X^T, b*A + c*A*A and a*X + P*X are all instances of it (see GemmArgs).
 #include "fm_internal.h"
+#include <atomic>
 #include <cstdlib>
 
 namespace fm {
 
 constexpr int ROW_BYTES = 128;         // one LDS row: the k extent of a stage, 64 16-bit or 32 32-bit elements
 
-// 16-byte chunk c of LDS row r lives at chunk position c ^ swz(r).  Any 8 consecutive rows get 8
-// distinct positions within a 128-byte bank group and any 16 consecutive rows get 16 distinct
-// positions within 256 bytes, so a ds_read_b128 of one chunk column over 32 rows is conflict free.
-__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
-
 __device__ __forceinline__ uint32_t lds_off(int row, int chunk) {
   return (uint32_t)(row * ROW_BYTES + ((chunk ^ swz(row)) << 4));
-}
-
-// Upper-triangular tile index t (row-major over rows i, columns j >= i) -> (i, j).
-__device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
-  float fT = (float)(2 * T + 1);
-  int ii = (int)((fT - __builtin_sqrtf(fT * fT - 8.0f * (float)t)) * 0.5f);
-  if (ii < 0) ii = 0;
-  if (ii > T - 1) ii = T - 1;
-  // S(i) = number of tiles in rows < i
-  while (ii > 0 && (ii * T - (ii * (ii - 1)) / 2) > t) --ii;
-  while (ii + 1 < T && ((ii + 1) * T - ((ii + 1) * ii) / 2) <= t) ++ii;
-  i = ii;
-  j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
 }
 
 // ES: bytes per element (2 or 4).  A 16-byte chunk holds 16 / ES consecutive k.
@@ -274,10 +257,49 @@ int launch_gemm_general(GemmArgs a, hipStream_t stream) {
 
 int launch_gemm_nt(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
   if (a.batch < 1) a.batch = 1;
-  if (gemm_fast_eligible(a) && ws && ws_bytes >= gemm_fast_workspace_bytes(a.Ma, a.Nb, a.symmetric != 0))
-    return launch_gemm_fast(a, ws, ws_bytes, stream);
-  if (gemm_mid_eligible(a) && !std::getenv("FLASHMUON_NO_MID")) return launch_gemm_mid(a, stream);
+  if (gemm_fast_eligible(a)) {
+    // a workspace too small for this shape's schedule sends the problem down the slower paths
+    const int rc = launch_gemm_fast(a, ws, ws_bytes, stream);
+    if (rc != kErrWorkspace) return rc;
+  }
+  if (gemm_mid_eligible(a) && knob(kKnobNoMid) <= 0) return launch_gemm_mid(a, stream);
   return launch_gemm_general(a, stream);
+}
+
+// ---- knobs and device facts, read once ---------------------------------------------------------
+namespace {
+struct KnobState {
+  std::atomic<long long> v[kKnobCount];
+  KnobState() {
+    static const char* const names[kKnobCount] = {"FLASHMUON_GRID", "FLASHMUON_KSPLIT", "FLASHMUON_FAST_MIN_UNITS",
+                                                  "FLASHMUON_NO_MID"};
+    for (int i = 0; i < kKnobCount; ++i) {
+      const char* e = std::getenv(names[i]);
+      v[i].store(e ? std::atoll(e) : -1, std::memory_order_relaxed);
+    }
+  }
+};
+KnobState& knob_state() { static KnobState s; return s; }
+}  // namespace
+
+long long knob(int which) { return knob_state().v[which].load(std::memory_order_relaxed); }
+int set_knob(int which, long long value) {
+  if (which < 0 || which >= kKnobCount) return -1;
+  knob_state().v[which].store(value, std::memory_order_relaxed);
+  return 0;
+}
+
+int cu_count() {
+  constexpr int kMaxDev = 64;
+  static std::atomic<int> cached[kMaxDev];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
 }
 
 }  // namespace fm

@@ -1,6 +1,6 @@
 // Fast path of the bf16 (or fp16) NT contraction for gfx950: 256x256 output tiles, 4 waves (one per SIMD) of
 // 128x128 each, 64-wide k stages copied global -> LDS by the DMA form of global_load (no VGPR
-// staging), two LDS stages.
+// staging) into a ring of three stages of operand A and two of operand B.
 //
 // Schedule.  One workgroup per CU.  Tiles are taken in rounds of `grid` whole tiles: all workgroups
 // start a tile together and walk k in step, so the workgroups of one XCD, which hold a compact
@@ -20,12 +20,11 @@ constexpr int ROWB = BKF * 2;               // bytes per LDS row
 constexpr int OPER_BYTES = BM * ROWB;       // one operand stage: 32 KiB
 constexpr int PART_FLOATS = BM * BN;        // one fp32 partial tile
 constexpr int kMaxParts = 64;               // parts one tile can be cut into
-constexpr int kMaxSlots = 768;              // partial-tile slots the workspace holds (192 MiB)
+constexpr int kMaxSlots = 768;              // partial-tile slots a schedule may use (192 MiB)
+constexpr int kMaxGrid = 256;               // workgroups per launch: the XCD remap and the slot count assume no more
 constexpr int kMaxKsplit = 16;              // base parts per tile
 
 #define FM_LDS_ADDR(p) ((uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)(p)))
-
-__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 // One wave-wide global -> LDS copy of 16 bytes per lane: lane l lands at lds_base + 16*l.
 // The compiler does not see the LDS write, so every use is ordered by hand with
@@ -38,66 +37,95 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-__device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
-  float fT = (float)(2 * T + 1);
-  int ii = (int)((fT - __builtin_sqrtf(fT * fT - 8.0f * (float)t)) * 0.5f);
-  if (ii < 0) ii = 0;
-  if (ii > T - 1) ii = T - 1;
-  while (ii > 0 && (ii * T - (ii * (ii - 1)) / 2) > t) --ii;
-  while (ii + 1 < T && ((ii + 1) * T - ((ii + 1) * ii) / 2) <= t) ++ii;
-  i = ii;
-  j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
-}
-
 #define FM_MFMA(i, j, FA, FB) acc[i][j] = mfma_32x32x16<F16>(FA[i], FB[j], acc[i][j])
 
 struct Frag { bf16x8_t a[4], b[4]; };
 
-__device__ __forceinline__ void read_frags(Frag& f, const unsigned char* sa, const unsigned char* sb,
-                                           const uint32_t (&ao)[4], const uint32_t (&bo)[4], int ks) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) f.a[i] = *reinterpret_cast<const bf16x8_t*>(sa + (ao[i] ^ (ks << 5)));
-#pragma unroll
-  for (int j = 0; j < 4; ++j) f.b[j] = *reinterpret_cast<const bf16x8_t*>(sb + (bo[j] ^ (ks << 5)));
+// LDS during the main loop: three stages of operand A and two of operand B, 32 KiB each, in the
+// order A0 A1 B0 B1 A2.  Stage s of A sits in A slot s % 3, stage s of B in B slot s % 2.  A
+// ds_read takes a 16-bit immediate offset, so one address register reaches two neighbouring slots:
+// the fragment addresses are kept for the windows at 0 (A0, A1), 64 KiB (B0, B1) and 128 KiB (A2)
+// and no address arithmetic is left in the loop (every VALU instruction between two MFMAs delays
+// the second one by its own issue time).
+constexpr int A_SLOTS = 3, B_SLOTS = 2;
+__host__ __device__ constexpr int a_slot_off(int slot) { return slot == 2 ? 4 * OPER_BYTES : slot * OPER_BYTES; }
+__host__ __device__ constexpr int b_slot_off(int slot) { return (2 + slot) * OPER_BYTES; }
+
+// per-lane LDS byte addresses of the fragments: [window][fragment][k16 substep]
+struct FragAddr {
+  uint32_t a_lo[4][4];   // A rows, slots 0 and 1 (offset 0 / OPER_BYTES)
+  uint32_t a_hi[4][4];   // A rows, slot 2
+  uint32_t b[4][4];      // B rows, B slots 0 and 1 (offset 0 / OPER_BYTES from the window at 64 KiB)
+};
+
+template <int ASLOT>
+__device__ __forceinline__ bf16x8_t read_a(const unsigned char* smem, const FragAddr& fa, int i, int ks) {
+  if constexpr (ASLOT == 2) return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_hi[i][ks]);
+  else return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_lo[i][ks] + ASLOT * OPER_BYTES);
+}
+template <int BSLOT>
+__device__ __forceinline__ bf16x8_t read_b(const unsigned char* smem, const FragAddr& fa, int j, int ks) {
+  return *reinterpret_cast<const bf16x8_t*>(smem + fa.b[j][ks] + BSLOT * OPER_BYTES);
 }
 
-// 16 MFMAs of one k16 substep; the 8 fragment reads of the next substep ride on the first 8.
-template <bool F16>
+// one global -> LDS copy with the destination given as an offset from the wave's copy base
+__device__ __forceinline__ void dma16o(uint32_t voff, const void* sbase, uint32_t lds_base, int off) {
+  asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory");
+}
+
+// 16 MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The 8 fragment reads of the next
+// substep ride on the first 8, and copies Q0 .. Q1-1 of operand A of the stage two ahead (into the
+// A slot that the previous stage has left) go out between the others, so that the memory pipeline
+// sees an even stream of requests and each of these copies has almost two stages to land.
+template <bool F16, int ASLOT, int BSLOT, int KS, int Q0, int Q1>
 __device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
-                                      const unsigned char* sa, const unsigned char* sb,
-                                      const uint32_t (&ao)[4], const uint32_t (&bo)[4], int ks_next) {
-  read_frags(nxt, sa, sb, ao, bo, ks_next);
-#pragma unroll
-  for (int q = 0; q < 16; ++q) FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
-#pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-  }
-  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-  __builtin_amdgcn_sched_barrier(0);
-}
-
-// Last substep of a stage.  After the barrier every wave holds its last fragments of this stage in
-// registers and the other stage has landed, so the 16 MFMAs run interleaved with the DMA that
-// refills this stage (16 copies) and with the first fragment reads of the other stage.
-template <bool F16>
-__device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
-                                           const unsigned char* nsa, const unsigned char* nsb,
-                                           const uint32_t (&ao)[4], const uint32_t (&bo)[4],
-                                           const uint32_t (&voA)[8], const uint32_t (&voB)[8],
-                                           const bf16_t* gA, const bf16_t* gB, uint32_t ldsA, uint32_t ldsB) {
-  wait_vmcnt<0>();
-  __syncthreads();
+                                      const unsigned char* smem, const FragAddr& fa,
+                                      const uint32_t (&voA)[8], const bf16_t* gA, uint32_t ldsw) {
+  constexpr int AFREE = (ASLOT + 2) % 3;
 #pragma unroll
   for (int q = 0; q < 16; ++q) {
-    if (q < 8) dma16(voA[q], gA, ldsA + q * 4096);
-    else dma16(voB[q - 8], gB, ldsB + (q - 8) * 4096);
-    if (q < 4) nxt.a[q] = *reinterpret_cast<const bf16x8_t*>(nsa + ao[q]);
-    else if (q < 8) nxt.b[q - 4] = *reinterpret_cast<const bf16x8_t*>(nsb + bo[q - 4]);
+    if (q < 4) nxt.a[q] = read_a<ASLOT>(smem, fa, q, KS + 1);
+    else if (q < 8) nxt.b[q - 4] = read_b<BSLOT>(smem, fa, q - 4, KS + 1);
+    if (q >= 9 && ((q - 9) & 1) == 0 && Q0 + (q - 9) / 2 < Q1)
+      dma16o(voA[Q0 + (q - 9) / 2], gA, ldsw, a_slot_off(AFREE) + (Q0 + (q - 9) / 2) * 4096);
     FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
     __builtin_amdgcn_sched_barrier(0);
   }
+}
+
+// Last substep of a stage.  Before it every wave waits for its copies of the next stage (all but
+// the 8 newest, which belong to the stage after) and, at the barrier, for everybody else's; then
+// the 16 MFMAs run interleaved with the 8 copies of operand B two stages ahead, into the B slot
+// this stage has just left, and with the first fragment reads of the next stage.
+template <bool F16, int ASLOT, int BSLOT>
+__device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
+                                           const unsigned char* smem, const FragAddr& fa,
+                                           const uint32_t (&voB)[8], const bf16_t* gB, uint32_t ldsw) {
+  constexpr int ANEXT = (ASLOT + 1) % 3, BNEXT = BSLOT ^ 1;
+  // (the fragment reads of this stage were issued a substep ago; lgkmcnt(0) makes it formal that
+  // nobody still reads the slots that are about to be refilled)
+  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    if ((q & 1) == 0) dma16o(voB[q >> 1], gB, ldsw, b_slot_off(BSLOT) + (q >> 1) * 4096);
+    if (q < 4) nxt.a[q] = read_a<ANEXT>(smem, fa, q, 0);
+    else if (q < 8) nxt.b[q - 4] = read_b<BNEXT>(smem, fa, q - 4, 0);
+    FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// one k stage: the stage in (ASLOT, BSLOT) is multiplied, operand A of the stage two ahead is
+// copied during the first three substeps and operand B of it during the last
+template <bool F16, int ASLOT, int BSLOT>
+__device__ __forceinline__ void stage(f32x16_t (&acc)[4][4], Frag& f0, Frag& f1, const unsigned char* smem,
+                                      const FragAddr& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                      const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
+  phase<F16, ASLOT, BSLOT, 0, 0, 3>(acc, f0, f1, smem, fa, voA, nA, ldsw);
+  phase<F16, ASLOT, BSLOT, 1, 3, 6>(acc, f1, f0, smem, fa, voA, nA, ldsw);
+  phase<F16, ASLOT, BSLOT, 2, 6, 8>(acc, f0, f1, smem, fa, voA, nA, ldsw);
+  tail_phase<F16, ASLOT, BSLOT>(acc, f1, f0, smem, fa, voB, nB, ldsw);
 }
 
 // ---- the part of a tile after the main loop -----------------------------------------------------
@@ -117,7 +145,7 @@ constexpr int QF_FLOATS = 128 * QF_PITCH;                 // 18432 bytes
 constexpr int QE_BYTES = 32 * 256;                        // one E buffer: 32 rows of 128 bf16
 constexpr int EPI_WAVE_BYTES = QF_FLOATS * 4 + 2 * QE_BYTES + 512;   // 35328
 constexpr int QUARTER_FLOATS = 128 * 32;                  // fp32 values of a quarter (partial tiles)
-constexpr int SMEM_BYTES = 4 * EPI_WAVE_BYTES;            // 141312 >= the 131072 of the operand stages
+constexpr int SMEM_BYTES = 5 * OPER_BYTES;                // 163840: the operand ring; the staging needs 4 * EPI_WAVE_BYTES = 141312
 
 struct EpiLds {
   float* F;
@@ -343,10 +371,6 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // two operand stages (A0 B0 A1 B1, 32 KiB each) during the main loop, the accumulator staging of
   // the four waves afterwards
   __shared__ __align__(1024) unsigned char smem[SMEM_BYTES];
-  unsigned char* const sA0 = smem;
-  unsigned char* const sB0 = smem + OPER_BYTES;
-  unsigned char* const sA1 = smem + 2 * OPER_BYTES;
-  unsigned char* const sB1 = smem + 3 * OPER_BYTES;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -360,17 +384,22 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     if (w < chunk * 8) w = (w & 7) * chunk + (w >> 3);
   }
 
-  const uint32_t lA0 = FM_LDS_ADDR(sA0) + wave * 1024, lB0 = FM_LDS_ADDR(sB0) + wave * 1024;
-  const uint32_t lA1 = FM_LDS_ADDR(sA1) + wave * 1024, lB1 = FM_LDS_ADDR(sB1) + wave * 1024;
+  const uint32_t ldsw = FM_LDS_ADDR(smem) + wave * 1024;   // where this wave's copies land inside a slot
 
-  // per-lane fragment offsets inside an operand stage (row = lane % 32, k half = lane / 32)
-  uint32_t ao[4], bo[4];
+  // per-lane fragment addresses (row = lane % 32 of the fragment's 32 rows, k half = lane / 32)
+  FragAddr fa;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int ra = wm * 128 + i * 32 + (lane & 31);
-    ao[i] = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
     const int rb = wn * 128 + i * 32 + (lane & 31);
-    bo[i] = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
+    const uint32_t ao = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
+    const uint32_t bo = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      fa.a_lo[i][ks] = ao ^ (ks << 5);
+      fa.a_hi[i][ks] = (ao ^ (ks << 5)) + a_slot_off(2);
+      fa.b[i][ks] = (bo ^ (ks << 5)) + b_slot_off(0);
+    }
   }
 
   for (int round = 0; round <= p.rounds; ++round) {
@@ -417,43 +446,51 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     // ---- main loop over k stages kb .. ke-1 ----------------------------------------------------
     {
       Frag f0, f1;
-      const int k1 = n > 1 ? 1 : 0;
+      // stages past the end are the last stage again (into slots nobody reads), so that the number
+      // of copies in flight is the same at every wait
+      const int last = n - 1;
+      const int k1 = last < 1 ? last : 1;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) { dma16(voA[q], gA, lA0 + q * 4096); dma16(voB[q], gB, lB0 + q * 4096); }
+      for (int q = 0; q < 8; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        dma16(voA[q], gA + k1 * BKF, lA1 + q * 4096);
-        dma16(voB[q], gB + k1 * BKF, lB1 + q * 4096);
-      }
+      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, b_slot_off(0) + q * 4096);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, b_slot_off(1) + q * 4096);
       wait_vmcnt<16>();
       __syncthreads();
-      read_frags(f0, sA0, sB0, ao, bo, 0);
-      // stages go through the loop in pairs (a loop with a second exit in the middle makes the
-      // register allocator give up on keeping the accumulators in place); an odd last stage follows
-      int it = 0;
-      for (; it + 2 <= n; it += 2) {
-        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 1);
-        phase<F16>(acc, f1, f0, sA0, sB0, ao, bo, 2);
-        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 3);
-        {
-          const int kn = (it + 2 < n) ? it + 2 : n - 1;
-          tail_phase<F16>(acc, f1, f0, sA1, sB1, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA0, lB0);
-        }
-        phase<F16>(acc, f0, f1, sA1, sB1, ao, bo, 1);
-        phase<F16>(acc, f1, f0, sA1, sB1, ao, bo, 2);
-        phase<F16>(acc, f0, f1, sA1, sB1, ao, bo, 3);
-        {
-          const int kn = (it + 3 < n) ? it + 3 : n - 1;
-          tail_phase<F16>(acc, f1, f0, sA0, sB0, ao, bo, voA, voB, gA + kn * BKF, gB + kn * BKF, lA1, lB1);
-        }
-      }
-      if (it < n) {   // one stage left: it sits in stage 0 and its first fragments are in f0
-        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 1);
-        phase<F16>(acc, f1, f0, sA0, sB0, ao, bo, 2);
-        phase<F16>(acc, f0, f1, sA0, sB0, ao, bo, 3);
 #pragma unroll
-        for (int q = 0; q < 16; ++q) FM_MFMA(q >> 2, q & 3, f1.a, f1.b);
+      for (int q = 0; q < 4; ++q) { f0.a[q] = read_a<0>(smem, fa, q, 0); f0.b[q] = read_b<0>(smem, fa, q, 0); }
+      // the slots come round every 6 stages
+#define FM_STAGE(AS, BS, S)                                                                      \
+      {                                                                                          \
+        const int kn = (S) + 2 < last ? (S) + 2 : last;                                          \
+        stage<F16, AS, BS>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
       }
+      int s = 0;
+      for (; s + 6 <= n; s += 6) {
+        FM_STAGE(0, 0, s)
+        FM_STAGE(1, 1, s + 1)
+        FM_STAGE(2, 0, s + 2)
+        FM_STAGE(0, 1, s + 3)
+        FM_STAGE(1, 0, s + 4)
+        FM_STAGE(2, 1, s + 5)
+      }
+      if (s < n) {
+        FM_STAGE(0, 0, s)
+        if (s + 1 < n) {
+          FM_STAGE(1, 1, s + 1)
+          if (s + 2 < n) {
+            FM_STAGE(2, 0, s + 2)
+            if (s + 3 < n) {
+              FM_STAGE(0, 1, s + 3)
+              if (s + 4 < n) FM_STAGE(1, 0, s + 4)
+            }
+          }
+        }
+      }
+#undef FM_STAGE
       wait_vmcnt<0>();
       __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
     }
@@ -700,15 +737,17 @@ static int auto_ksplit(long long num_tiles, int nk, int grid) {
   return ksplit;
 }
 
-// the schedule for `num_tiles` tiles of `nk` k stages
-static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
-  int grid = 256;                                   // one workgroup per CU (138 KiB of LDS each)
-  if (const char* e = std::getenv("FLASHMUON_GRID")) grid = std::atoi(e);   // tuning aid
-  if (grid > 256) grid = 256;
+// the schedule for `num_tiles` tiles of `nk` k stages; `max_slots` partial-tile slots are there
+static void fast_schedule(int num_tiles, int nk, long long max_slots, FastArgs& f) {
+  int grid = cu_count();                            // one workgroup per CU (160 KiB of LDS each)
+  if (grid > kMaxGrid) grid = kMaxGrid;
+  const long long kg = knob(kKnobGrid);             // tuning aid
+  if (kg > 0 && kg < grid) grid = (int)kg;
   int ksplit = auto_ksplit(num_tiles, nk, grid);
-  if (const char* e = std::getenv("FLASHMUON_KSPLIT")) ksplit = std::atoi(e);   // tuning aid
+  const long long kk = knob(kKnobKsplit);           // tuning aid
+  if (kk > 0) ksplit = (int)kk;
   if (ksplit < 1 || ksplit > nk || ksplit > kMaxKsplit) ksplit = 1;
-  if (ksplit > 1 && (int64_t)num_tiles * ksplit + grid > kMaxSlots) ksplit = 1;   // slots: items + rem * split
+  if (ksplit > 1 && (long long)num_tiles * ksplit + grid > max_slots) ksplit = 1;   // slots: items + rem * split
   const int items = num_tiles * ksplit;
   if (grid > items) grid = items;                   // rem * split never exceeds the grid below
   if (grid < 1) grid = 1;
@@ -723,6 +762,9 @@ static void fast_schedule(int num_tiles, int nk, FastArgs& f) {
     if (s > base_stages) s = base_stages;
     if (s > 16) s = 16;                             // bounds the partial-tile traffic
     if (s > kMaxParts / ksplit) s = kMaxParts / ksplit;
+    // what the workspace holds; with ksplit == 1 and no room the last round runs whole tiles
+    const long long room = max_slots - (ksplit > 1 ? (long long)f.rounds * grid : 0);
+    if ((long long)f.rem * s > room) s = (int)(room / f.rem);
     f.split = s < 1 ? 1 : s;
   }
   f.tail_slot0 = ksplit > 1 ? f.rounds * grid : 0;
@@ -760,17 +802,18 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   const long long tm = a.Ma / BM, tn = a.Nb / BN;
   const long long tiles = (a.symmetric ? tm * (tm + 1) / 2 : tm * tn) * (a.batch < 1 ? 1 : a.batch);
   const int nk = a.Kc / BKF;
-  // FLASHMUON_FAST_MIN_UNITS replaces the choice below by a threshold on (tile, k-stage) units,
+  // the FAST_MIN_UNITS knob replaces the choice below by a threshold on (tile, k-stage) units,
   // e.g. 0 to exercise this path on small inputs
-  if (const char* e = std::getenv("FLASHMUON_FAST_MIN_UNITS")) return tiles * nk >= std::atoll(e);
+  if (knob(kKnobFastMinUnits) >= 0) return tiles * nk >= knob(kKnobFastMinUnits);
   // More tiles than workgroups: rounds of large tiles.  Otherwise it is one round of 256x256 tiles
   // on some of the CUs against one or more waves of 128x128 tiles on all of them; estimate both in
   // microseconds from the measured cost of a k stage and of a tile's epilogue on each path.
-  if (tiles > 256) return true;
-  const int ksplit = auto_ksplit(tiles, nk, 256);
+  const int cus = cu_count() < kMaxGrid ? cu_count() : kMaxGrid;
+  if (tiles > cus) return true;
+  const int ksplit = auto_ksplit(tiles, nk, cus);
   const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
   const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
-  const double t_small = (double)((small_tiles + 255) / 256) * (nk * 0.55 + 6.0);
+  const double t_small = (double)((small_tiles + cus - 1) / cus) * (nk * 0.55 + 6.0);
   return t_large < t_small;
 }
 
@@ -786,10 +829,26 @@ int launch_gemm_mid(GemmArgs a, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric) {
-  (void)Ma; (void)Nb; (void)symmetric;
-  // items of full rounds (only when tiles are cut: fewer than 2 * 256 of them) + rem * split <= 256
-  return (size_t)kMaxSlots * PART_FLOATS * sizeof(float);
+size_t gemm_fast_workspace_bytes(int Ma, int Nb, int batch) {
+  if (Ma < BM || Nb < BN || Ma % BM != 0 || Nb % BN != 0) return 0;   // never on this path
+  if (batch < 1) batch = 1;
+  const long long tm = Ma / BM, tn = Nb / BN;
+  // a square output may be a symmetric product (fewer tiles) or a general one: take the larger need
+  long long need = 0;
+  for (int sym = 0; sym < (Ma == Nb ? 2 : 1); ++sym) {
+    const long long tiles = (sym ? tm * (tm + 1) / 2 : tm * tn) * batch;
+    long long slots;
+    if (tiles * 5 < (long long)kMaxGrid * 3) {
+      // every tile may be cut into base parts (auto_ksplit), and the left-over items once more
+      slots = tiles * kMaxKsplit + kMaxGrid;
+      if (slots > kMaxSlots) slots = kMaxSlots;
+    } else {
+      // only the items left after the last full round are cut, into at most one round of parts
+      slots = kMaxGrid;
+    }
+    if (slots > need) need = slots;
+  }
+  return (size_t)need * PART_FLOATS * sizeof(float);
 }
 
 int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
@@ -800,13 +859,12 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   FastArgs f;
   f.g = a;
   f.nk = a.Kc / BKF;
-  fast_schedule(a.num_tiles, f.nk, f);
+  const long long have = ws ? (long long)(ws_bytes / (PART_FLOATS * sizeof(float))) : 0;
+  fast_schedule(a.num_tiles, f.nk, have < kMaxSlots ? have : kMaxSlots, f);
   f.partials = static_cast<float*>(ws);
   const int slots = f.tail_slot0 + f.rem * f.split;
   const int reduce_tiles = a.num_tiles - f.reduce_tile0;
-  if (reduce_tiles > 0 && (!ws || slots > kMaxSlots || ws_bytes < (size_t)slots * PART_FLOATS * sizeof(float) ||
-                           f.ksplit * f.split > kMaxParts))
-    return -1;
+  if (reduce_tiles > 0 && (slots > have || f.ksplit * f.split > kMaxParts)) return kErrWorkspace;
   if (a.elem == kElemF16) {
     hipLaunchKernelGGL(gemm_nt_rounds_kernel<true>, dim3(f.grid), dim3(256), 0, stream, f);
     if (reduce_tiles > 0)

@@ -15,6 +15,37 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 constexpr int kMaxBatch = 16;         // matrices per batched launch
 constexpr int kElemBf16 = 0, kElemF16 = 1, kElemF32 = 2;
 
+// what the launch functions return besides hipError_t values (which are >= 0)
+constexpr int kErrWorkspace = -2;     // the schedule needs more partial-tile slots than the workspace holds
+
+// Tuning knobs (fm_set_knob, include/flashmuon.h); the FLASHMUON_* environment variables of the same
+// names give their initial values, read once when the library is first used.  A negative value
+// means "decide automatically".
+constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobCount = 4;
+long long knob(int which);
+int set_knob(int which, long long value);
+// compute units of the current device (queried once per device)
+int cu_count();
+
+// 16-byte chunk c of a 128-byte LDS row r lives at chunk position c ^ swz(r).  Any 8 consecutive
+// rows get 8 distinct positions within a 128-byte bank group and any 16 consecutive rows get 16
+// distinct positions within 256 bytes, so a ds_read_b128 of one chunk column over 32 rows is
+// conflict free.
+__device__ __forceinline__ int swz(int row) { return (row ^ (row >> 3)) & 7; }
+
+// Upper-triangular tile index t (row-major over rows i, columns j >= i) -> (i, j).
+__device__ __forceinline__ void tri_decode(int t, int T, int& i, int& j) {
+  float fT = (float)(2 * T + 1);
+  int ii = (int)((fT - __builtin_sqrtf(fT * fT - 8.0f * (float)t)) * 0.5f);
+  if (ii < 0) ii = 0;
+  if (ii > T - 1) ii = T - 1;
+  // S(i) = number of tiles in rows < i
+  while (ii > 0 && (ii * T - (ii * (ii - 1)) / 2) > t) --ii;
+  while (ii + 1 < T && ((ii + 1) * T - ((ii + 1) * ii) / 2) <= t) ++ii;
+  i = ii;
+  j = ii + (t - (ii * T - (ii * (ii - 1)) / 2));
+}
+
 // The GEMM kernels exist for two 16-bit element types with the same memory layout; pointers are
 // typed bf16_t in both cases and F16 says what the bits mean.
 template <bool F16>
@@ -87,7 +118,10 @@ __host__ __device__ inline GemmArgs batch_view(const GemmArgs& g, int b) {
 int launch_gemm_nt(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
 int launch_gemm_general(GemmArgs args, hipStream_t stream);
 bool gemm_fast_eligible(const GemmArgs& a);
-size_t gemm_fast_workspace_bytes(int Ma, int Nb, bool symmetric);
+// bytes of fp32 partial tiles the 256x256 path can need for `batch` Ma x Nb outputs, whatever k is
+// (0 when no schedule of this shape cuts a tile)
+size_t gemm_fast_workspace_bytes(int Ma, int Nb, int batch);
+// kErrWorkspace when the schedule needs more than ws holds
 int launch_gemm_fast(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
 bool gemm_mid_eligible(const GemmArgs& a);
 int launch_gemm_mid(GemmArgs args, hipStream_t stream);

@@ -39,14 +39,22 @@ def matmul_transpose_assign(d_in, d_out):
         d_in = d_in.contiguous()
     ldx = d_in.stride(0) if K > 0 and M > 1 else max(K, 1)
     lib = _lib.load()
+    # an output whose strides fold two elements onto one address, or interleave rows and columns,
+    # is written through a dense temporary, as the reference's masked stores would fill it
+    rs, cs = (abs(d_out.stride(0)), abs(d_out.stride(1))) if M > 1 else (M, 1)
+    dst = d_out
+    if M > 1 and (min(rs, cs) == 0 or max(rs, cs) < M * min(rs, cs)):
+        dst = torch.empty((M, M), device=d_in.device, dtype=d_in.dtype)
     with torch.cuda.device(d_in.device):
         need = 0 if d_in.dtype == torch.float32 else lib.fm_gemm_workspace_bytes(M, M)
-        ws, ws_bytes = _lib.workspace(need, d_in.device)
-        st = getattr(lib, entry)(d_in.data_ptr(), ldx, d_out.data_ptr(),
-                                 d_out.stride(0) if M > 1 else M, d_out.stride(1) if M > 1 else 1,
+        ws, ws_bytes = _lib.gemm_workspace(need, d_in.device)
+        st = getattr(lib, entry)(d_in.data_ptr(), ldx, dst.data_ptr(),
+                                 dst.stride(0) if M > 1 else M, dst.stride(1) if M > 1 else 1,
                                  M, K, ws.data_ptr() if ws is not None else None, ws_bytes,
                                  _lib.stream_ptr(d_in.device))
     _lib.check(entry, st)
+    if dst is not d_out:
+        d_out.copy_(dst)
 
 
 def matmul_transpose(d_in):

@@ -37,7 +37,8 @@ enum fm_status {
   FM_OK = 0,
   FM_ERR_NULL = 1,        /* a required pointer is NULL */
   FM_ERR_SHAPE = 2,       /* a dimension is negative, zero where forbidden, or inconsistent */
-  FM_ERR_STRIDE = 3,      /* a leading dimension is smaller than the row it must hold */
+  FM_ERR_STRIDE = 3,      /* a leading dimension is smaller than the row it must hold, or output
+                             strides that map two elements to one address */
   FM_ERR_DTYPE = 4,       /* dtype code not one of FM_BF16 / FM_F16 / FM_F32 */
   FM_ERR_ALIAS = 5,       /* an output overlaps an input it must not overlap */
   FM_ERR_WORKSPACE = 6,   /* ws is NULL or ws_bytes too small */
@@ -53,10 +54,26 @@ FM_API const char* fm_status_string(int status);
 /* Library version, "major.minor.patch". */
 FM_API const char* fm_version(void);
 
+/* Tuning knobs, for experiments and for tests that have to reach a particular schedule.  A
+ * negative value gives the decision back to the library.  The environment variables
+ * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS and FLASHMUON_NO_MID set the initial
+ * values; they are read once, when the library is first used, never per call.  No counterpart in
+ * the reference (its tuning is Triton's autotune table, flash_muon/matmul_transpose_triton.py:6-18).
+ */
+enum fm_knob {
+  FM_KNOB_GRID = 0,            /* workgroups per launch of the 256x256 schedule (at most one per CU) */
+  FM_KNOB_KSPLIT = 1,          /* base parts every tile of that schedule is cut into along k */
+  FM_KNOB_FAST_MIN_UNITS = 2,  /* take the 256x256 schedule when tiles * k-stages >= this (0: whenever the shape allows) */
+  FM_KNOB_NO_MID = 3           /* 1: never take the 128x128 copy-fed schedule */
+};
+FM_API int fm_set_knob(int knob, long long value);
+
 /* ---------------------------------------------------------------------------------------------
  * Scratch for the three GEMM-shaped entry points below, by the shape of their OUTPUT: (M, M) for
  * fm_syrk_bf16, fm_syrk_f16, fm_syrk_f32 and fm_syrk_poly_bf16, (M, K) for fm_gemm_axpby_bf16.  It holds the
- * fp32 partial tiles of output tiles whose k range is split over several workgroups.
+ * fp32 partial tiles of output tiles whose k range is split over several workgroups: 256 KiB per
+ * part, at most 256 parts (64 MiB) when the output has more 256x256 tiles than the GPU has CUs,
+ * at most 768 (192 MiB) below that, and 0 for shapes that never take that schedule.
  * The calls also run with ws == NULL (or a smaller ws) on a slower schedule that needs none.
  */
 FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
@@ -65,7 +82,9 @@ FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
  * Y = X * X^T, X is M x K bf16 (row stride ldx, unit column stride), Y is M x M bf16 with
  * arbitrary strides (ldy_row, ldy_col).  Only tiles on or above the diagonal are computed; every
  * tile above it is written twice, directly and mirrored, from the same accumulators, and Y == Y^T
- * holds bit for bit.  fp32 accumulation, one round-to-nearest-even to bf16.  Y must not overlap X.
+ * holds bit for bit.  fp32 accumulation, one round-to-nearest-even to bf16.  Y must not overlap X,
+ * and the larger of |ldy_row|, |ldy_col| must be at least M times the smaller (no two elements of
+ * Y at one address).
  * Replaces mmt_kernel + its launch: flash_muon/matmul_transpose_triton.py:20-75, 90-101.
  */
 FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,

@@ -20,3 +20,17 @@ def lib():
         from flash_muon_amd import build
         build.build(verbose=False)
     return _lib.load()
+
+
+KNOBS = {"FLASHMUON_GRID": 0, "FLASHMUON_KSPLIT": 1, "FLASHMUON_FAST_MIN_UNITS": 2, "FLASHMUON_NO_MID": 3}
+
+
+@pytest.fixture
+def knobs(lib):
+    """set(name, value) turns a tuning knob of the library (fm_set_knob) for the length of one test;
+    afterwards every knob is back on automatic."""
+    def set(name, value):
+        assert lib.fm_set_knob(KNOBS[name], int(value)) == 0
+    yield set
+    for k in KNOBS.values():
+        lib.fm_set_knob(k, -1)

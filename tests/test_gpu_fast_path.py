@@ -1,7 +1,6 @@
 """The 256x256 path of the GEMM-shaped kernels (rounds of whole tiles, tiles cut along k where the
 chip would otherwise idle).  It is chosen by shape (whole 256-tiles, k a multiple of 64, enough k
-stages to share out); FLASHMUON_FAST_MIN_UNITS=0 is set for every test here (the library reads it at
-each launch), so that small inputs take it too and the partial-tile hand-over is exercised with few,
+stages to share out); the FAST_MIN_UNITS knob is set to 0 for every test here (fm_set_knob), so that small inputs take it too and the partial-tile hand-over is exercised with few,
 many and uneven parts per tile.  Integer-valued inputs make every comparison bit-exact."""
 import pytest
 import torch
@@ -14,8 +13,8 @@ DEV = "cuda:0"
 
 
 @pytest.fixture(autouse=True)
-def _small_inputs_take_the_256_path(monkeypatch):
-    monkeypatch.setenv("FLASHMUON_FAST_MIN_UNITS", "0")
+def _small_inputs_take_the_256_path(knobs):
+    knobs("FLASHMUON_FAST_MIN_UNITS", 0)
 
 
 def _ints(shape, seed, lo=-2, hi=2):
@@ -46,10 +45,10 @@ def test_syrk_fast_integer_bit_exact(lib, M, K):
 
 @pytest.mark.parametrize("ksplit", [1, 2, 3, 4, 7, 16])
 @pytest.mark.parametrize("M,K", [(256, 448), (768, 1024), (1280, 8192), (4096, 1024)])
-def test_syrk_fast_forced_base_split(lib, monkeypatch, M, K, ksplit):
-    """Every tile cut into `ksplit` base parts along k (the library reads the variable at each launch):
+def test_syrk_fast_forced_base_split(lib, knobs, M, K, ksplit):
+    """Every tile cut into `ksplit` base parts along k (fm_set_knob):
     full rounds of partial tiles, a cut last round, and the second kernel over every tile."""
-    monkeypatch.setenv("FLASHMUON_KSPLIT", str(ksplit))
+    knobs("FLASHMUON_KSPLIT", ksplit)
     X = _ints((M, K), 7 * M + K + ksplit)
     want = _exact(X.double() @ X.double().T)
     Y = torch.full((M, M), 7.0, dtype=torch.bfloat16, device=DEV)
@@ -68,11 +67,11 @@ def test_syrk_fast_few_tiles_long_k(lib):
 
 @pytest.mark.parametrize("grid", [3, 8, 20, 24, 40, 57])
 @pytest.mark.parametrize("M,K,ksplit", [(1280, 512, 1), (2048, 1024, 1), (2048, 448, 2), (1792, 1344, 3)])
-def test_syrk_fast_small_grids(lib, monkeypatch, M, K, ksplit, grid):
-    """Few workgroups per round (the library reads FLASHMUON_GRID at each launch): several full
+def test_syrk_fast_small_grids(lib, knobs, M, K, ksplit, grid):
+    """Few workgroups per round (the GRID knob): several full
     rounds, last rounds of every fill, cut and uncut, on top of base parts."""
-    monkeypatch.setenv("FLASHMUON_GRID", str(grid))
-    monkeypatch.setenv("FLASHMUON_KSPLIT", str(ksplit))
+    knobs("FLASHMUON_GRID", grid)
+    knobs("FLASHMUON_KSPLIT", ksplit)
     X = _ints((M, K), 3 * M + K + grid)
     want = _exact(X.double() @ X.double().T)
     Y = torch.full((M, M), 7.0, dtype=torch.bfloat16, device=DEV)
@@ -81,8 +80,8 @@ def test_syrk_fast_small_grids(lib, monkeypatch, M, K, ksplit, grid):
 
 
 @pytest.mark.parametrize("grid", [8, 24, 40])
-def test_axpby_and_poly_fast_small_grids(lib, monkeypatch, grid):
-    monkeypatch.setenv("FLASHMUON_GRID", str(grid))
+def test_axpby_and_poly_fast_small_grids(lib, knobs, grid):
+    knobs("FLASHMUON_GRID", grid)
     M, K = 1024, 2304
     P = _ints((M, M), 41 + grid, -1, 1)
     X = _ints((M, K), 43 + grid)
@@ -99,8 +98,8 @@ def test_axpby_and_poly_fast_small_grids(lib, monkeypatch, grid):
 
 
 @pytest.mark.parametrize("ksplit", [2, 3])
-def test_axpby_fast_forced_base_split(lib, monkeypatch, ksplit):
-    monkeypatch.setenv("FLASHMUON_KSPLIT", str(ksplit))
+def test_axpby_fast_forced_base_split(lib, knobs, ksplit):
+    knobs("FLASHMUON_KSPLIT", ksplit)
     M, K = 768, 1536
     P = _ints((M, M), 31 + ksplit, -1, 1)
     X = _ints((M, K), 37 + ksplit)

@@ -68,13 +68,13 @@ def test_axpby_integer_bit_exact(lib, M, K):
     assert torch.equal(only_x.cpu(), (2 * X.double() + P.double() @ X.double()).float().bfloat16())
 
 
-def test_agrees_with_the_general_path_on_gaussian_input(lib, monkeypatch):
+def test_agrees_with_the_general_path_on_gaussian_input(lib, knobs):
     """Same bf16 input through this path and, with it switched off, through the general tiled
     path: both are one rounding of an fp32 sum, so they agree to within that rounding."""
     g = torch.Generator().manual_seed(5)
     X = torch.randn(1024, 2048, generator=g).bfloat16().to(DEV)
     mid = gpu_util.syrk(lib, X)
-    monkeypatch.setenv("FLASHMUON_NO_MID", "1")
+    knobs("FLASHMUON_NO_MID", 1)
     gen = gpu_util.syrk(lib, X)
     ref = X.float() @ X.float().T
     for Y in (mid, gen):

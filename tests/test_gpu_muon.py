@@ -26,6 +26,8 @@ def _device_params(ps, gs):
     out = []
     for p, g in zip(ps, gs):
         q = torch.nn.Parameter(p.clone().to(DEV))
+        if g.dtype != p.dtype and hasattr(q, "grad_dtype"):
+            q.grad_dtype = None          # an fp32 parameter with a bf16 gradient
         q.grad = g.clone().to(DEV)
         out.append(q)
     return out
