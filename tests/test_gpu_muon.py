@@ -122,8 +122,9 @@ def test_groups_state_dict_and_missing_grad():
     params = _device_params(ps, gs)
     opt = Muon(params, lr=LR, momentum=MU, rank=0, world_size=1)
     groups = opt.param_groups
-    assert [g["params"][0].numel() for g in groups] == [2048, 4096]
-    assert len(groups[1]["params"]) == 3
+    # one group per numel, in the iteration order of the reference's set expression (muon.py:68)
+    assert [g["params"][0].numel() for g in groups] == list({p.numel() for p in params}) == [4096, 2048]
+    assert len(groups[0]["params"]) == 3 and len(groups[1]["params"]) == 1
     for g in groups:
         assert set(g.keys()) >= {"params", "update_buffer", "update_buffer_views", "lr", "weight_decay",
                                  "momentum", "nesterov", "ns_steps"}
