@@ -2,6 +2,7 @@
 // Newton-Schulz composition.  No torch types, no allocation, no synchronisation.
 #include "../../include/flashmuon.h"
 #include "fm_internal.h"
+#include <atomic>
 
 using namespace fm;
 
@@ -49,6 +50,30 @@ NsLayout ns_layout(int batch, int rows, int cols) {
   l.gemm = take(g1 > g2 ? g1 : g2);
   l.total = off;
   return l;
+}
+
+// ---- scratch of fm_syrk_bf16_static -------------------------------------------------------------
+// 256 partial tiles of 256 KiB: what the 256x256 schedule needs at most when it cuts only the items
+// of its last round (more than that only buys a deeper k split of outputs with few tiles, which
+// this entry point then does without).  Every GPU the library runs on holds its own copy of the
+// array, at its own address, until the process ends.
+constexpr size_t kStaticScratchBytes = (size_t)256 * 256 * 256 * sizeof(float);   // 64 MiB
+static __device__ __align__(256) unsigned char fm_static_scratch[kStaticScratchBytes];
+
+// device address of the array on the current device, looked up once per device (in host code the
+// array's name is only a handle for this lookup, never an address a kernel could use)
+int static_scratch(void** out) {
+  constexpr int kMaxDev = 64;
+  static std::atomic<void*> per_device[kMaxDev];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return FM_ERR_LAUNCH;
+  void* p = per_device[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(fm_static_scratch)) != hipSuccess || !p) return FM_ERR_LAUNCH;
+    per_device[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return FM_OK;
 }
 
 }  // namespace
@@ -117,6 +142,15 @@ static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64
 int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
                  void* ws, size_t ws_bytes, fm_stream_t stream) {
   return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, ws, ws_bytes, stream, kElemBf16);
+}
+
+int fm_syrk_bf16_static(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
+                        fm_stream_t stream) {
+  if (M > FM_STATIC_MAX_M || K > FM_STATIC_MAX_K) return FM_ERR_SHAPE;
+  void* scratch = nullptr;
+  const int rc = static_scratch(&scratch);
+  if (rc != FM_OK) return rc;
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, scratch, kStaticScratchBytes, stream, kElemBf16);
 }
 
 int fm_syrk_f16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,

@@ -90,6 +90,22 @@ FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
 FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
                  int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
 
+/* fm_syrk_bf16 for callers that cannot allocate or hand over scratch memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments and results as fm_syrk_bf16 minus ws / ws_bytes: the partial tiles go
+ * to a 64 MiB array that the library holds in the device memory of every GPU it is used on, from the
+ * first use until the process ends.  Nothing is allocated, freed or synchronised; the first call on
+ * a device looks the array's address up (do that once outside a graph capture).
+ * Limits: M <= FM_STATIC_MAX_M and K <= FM_STATIC_MAX_K, otherwise FM_ERR_SHAPE.  All calls on one
+ * GPU share the array, which keeps the last call's contents (nothing in it has to start at zero:
+ * every part is written before it is read): calls that overlap in time on one GPU, i.e. on
+ * different streams, race with each other and must be ordered by the caller.
+ */
+#define FM_STATIC_MAX_M 65536
+#define FM_STATIC_MAX_K 1048576
+FM_API int fm_syrk_bf16_static(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
+                        int M, int K, fm_stream_t stream);
+
 /* The same product for fp16 X and Y (the reference's kernel takes its element type from the
  * input: flash_muon/matmul_transpose_triton.py:63): fp32 accumulation, one round-to-nearest-even
  * to fp16, same arguments and schedule.
