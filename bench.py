@@ -45,6 +45,37 @@ def _time_gpu(fn, steps, warmup, torch):
     return start.elapsed_time(end) / steps   # ms per call
 
 
+def _mfma_probe(torch):
+    """Sustained rate and clock of MFMA-only work (fm_probe_mfma_peak), on zeros and on N(0,1) bf16
+    operands: about 150 ms of back-to-back launches each, the second half timed."""
+    from flash_muon_amd import _lib
+    lib = _lib.load()
+    blocks, iters, launches = 256, 256, 480
+    sink = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
+    clocks = torch.zeros(blocks * 2, dtype=torch.int64, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(1)
+    out = {}
+    for name, ops in (("zeros", torch.zeros(blocks * 256 * 64, dtype=torch.bfloat16, device="cuda")),
+                      ("gaussian", torch.randn(blocks * 256 * 64, generator=g, device="cuda").bfloat16())):
+        st = _lib.stream_ptr("cuda")
+        lib.fm_probe_mfma_peak(ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        lib.fm_probe_mfma_peak(ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st)
+        e0.record()
+        rc = lib.fm_probe_mfma_peak(ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st)
+        e1.record()
+        torch.cuda.synchronize()
+        assert rc == 0
+        ms = e0.elapsed_time(e1) / (launches // 2)
+        c = clocks.view(blocks, 2).double().mean(0)
+        flop = blocks * 4 * iters * 64 * 32768.0
+        out[name] = {"tflops": flop / ms / 1e9, "ms_per_launch": ms, "shader_cycles": float(c[0]),
+                     "realtime_ticks_100mhz": float(c[1]), "clock_ghz": float(c[0] / c[1] / 10.0),
+                     "mfma_issue_fraction": iters * 64 * 32 / float(c[0])}
+    return out
+
+
 def _cpu_baseline(X, torch, ns=True, full=False):
     """torch fp32 X @ X.T on the host (the reference's own baseline, benchmark.py:20-21)."""
     from oracle import oracle
@@ -171,6 +202,9 @@ def main():
     ap.add_argument("--cpu-full", action="store_true",
                     help="also time the CPU oracle on Newton-Schulz 8192^2 and on one Llama-7B layer of "
                          "Muon.step (about a minute of CPU work)")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="only run the MFMA-only loop on zeros and on N(0,1) operands and print its sustained "
+                         "TFLOP/s and shader clock: the ceiling the power cap sets for matrix work")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 128 MiB device-to-device copy, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -187,6 +221,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
+    if args.mfma_probe:
+        print(json.dumps({"mfma_probe": _mfma_probe(torch)}))
+        return
 
     X = synthetic.gaussian_bf16(DIM, DIM, DIM)
     Xd = X.cuda()

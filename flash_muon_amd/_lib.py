@@ -49,6 +49,7 @@ SIGNATURES = {
     "fm_weight_update": (_i32, [_vp, _i32, _vp, _i64, _f32, _f32, _vp]),
     "fm_momentum_nesterov_batched": (_i32, [_vp, _vp, _i32, _i32, _i64, _f32, _f32, _i32, _vp]),
     "fm_weight_update_batched": (_i32, [_vp, _i32, _vp, _i32, _i64, _f32, _f32, _vp]),
+    "fm_probe_mfma_peak": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp]),
 }
 
 _lib = None

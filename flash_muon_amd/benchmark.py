@@ -2,10 +2,13 @@
 reference prints (benchmark.py:49-85): square bf16 inputs of 1024 .. 8192, 25 warm-up calls, 100
 timed calls between device events.
 
-    python -m flash_muon_amd.benchmark [--dims 1024 2048 4096 8192] [--warmup 25] [--rep 100]
+    python -m flash_muon_amd.benchmark [--dims 1024 2048 4096 8192] [--warmup 25] [--rep 100] [--no-compile]
 
 Two tables: `matmul_transpose` against `G @ G.T`, and `fast_newtonschulz` (5 steps) against the same
-iteration written with torch operators (benchmark.py:20-47).  torch's GEMMs go to the vendor BLAS.
+iteration written with torch operators (benchmark.py:20-47), each with the reference's three
+columns: this library, the torch baseline, and `torch.compile(baseline)` (benchmark.py:52-53).
+torch's GEMMs go to the vendor BLAS; the compiled column reads n/a where torch.compile cannot
+build the function on this machine (the reason is printed once).
 """
 import argparse
 
@@ -50,16 +53,26 @@ def _time(fn, x, warmup, rep):
     return start.elapsed_time(stop) / rep
 
 
-def run(name, impl, baseline, dims, warmup, rep):
+def run(name, impl, baseline, dims, warmup, rep, with_compiled=True):
     device = torch.cuda.get_device_name(torch.cuda.current_device())
+    compiled = torch.compile(baseline) if with_compiled else None
     rows = []
     for dim in dims:
         x = torch.randn(dim, dim, device="cuda").bfloat16()
-        rows.append((device, dim, _time(impl, x, warmup, rep), _time(baseline, x, warmup, rep)))
+        t_impl, t_base, t_comp = _time(impl, x, warmup, rep), _time(baseline, x, warmup, rep), None
+        if compiled is not None:
+            try:
+                t_comp = _time(compiled, x, warmup, rep)
+            except Exception as e:   # no working code generator on this machine: say so, once
+                print("torch.compile(%s) is not available here: %s: %s" % (baseline.__name__, type(e).__name__,
+                                                                            str(e).splitlines()[0][:200]))
+                compiled = None
+        rows.append((device, dim, t_impl, t_base, t_comp))
     print("\nbenchmark %s:" % name)
-    print("%-28s %6s %12s %12s %9s" % ("device", "dim", "flash(ms)", "torch(ms)", "speedup"))
-    for device, dim, t_impl, t_base in rows:
-        print("%-28s %6d %12.6f %12.6f %8.2fx" % (device[:28], dim, t_impl, t_base, t_base / t_impl))
+    print("%-28s %6s %12s %12s %13s %9s" % ("device", "dim", "flash(ms)", "torch(ms)", "compiled(ms)", "speedup"))
+    for device, dim, t_impl, t_base, t_comp in rows:
+        comp = "%13.6f" % t_comp if t_comp is not None else "%13s" % "n/a"
+        print("%-28s %6d %12.6f %12.6f %s %8.2fx" % (device[:28], dim, t_impl, t_base, comp, t_base / t_impl))
     return rows
 
 
@@ -68,11 +81,12 @@ def main(argv=None):
     ap.add_argument("--dims", type=int, nargs="+", default=[1024, 2048, 4096, 8192])
     ap.add_argument("--warmup", type=int, default=25)
     ap.add_argument("--rep", type=int, default=100)
+    ap.add_argument("--no-compile", action="store_true", help="leave the torch.compile column out")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit("flash_muon_amd.benchmark needs a GPU")
-    run("matmul transpose", matmul_transpose, torch_matmul_transpose, args.dims, args.warmup, args.rep)
-    run("zeropower", fast_newtonschulz, torch_newtonschulz5, args.dims, args.warmup, args.rep)
+    run("matmul transpose", matmul_transpose, torch_matmul_transpose, args.dims, args.warmup, args.rep, not args.no_compile)
+    run("zeropower", fast_newtonschulz, torch_newtonschulz5, args.dims, args.warmup, args.rep, not args.no_compile)
 
 
 if __name__ == "__main__":

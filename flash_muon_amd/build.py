@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJDIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libflashmuon_hip.so")
-SOURCES = ["fm_gemm.hip", "fm_gemm_fast.hip", "fm_elementwise.hip", "fm_api.hip"]
+SOURCES = ["fm_gemm.hip", "fm_gemm_fast.hip", "fm_elementwise.hip", "fm_api.hip", "fm_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -39,7 +39,7 @@ def _compile(src):
 
 def build(verbose=True):
     os.makedirs(OBJDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
         objs = list(ex.map(_compile, SOURCES))
     tmp = LIB_PATH + ".tmp"
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]

@@ -12,7 +12,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
-constexpr int kMaxBatch = 16;         // matrices per batched launch
+constexpr int kMaxBatch = 32;         // matrices per batched launch
 constexpr int kElemBf16 = 0, kElemF16 = 1, kElemF32 = 2;
 
 // what the launch functions return besides hipError_t values (which are >= 0)

@@ -26,7 +26,7 @@ def _rows_unit_stride(G):
     return G.contiguous()
 
 
-MAX_BATCH = 16  # kMaxBatch of the library: matrices per batched launch
+MAX_BATCH = 32  # kMaxBatch of the library: matrices per batched launch
 
 
 def _newtonschulz_into(Gs, outs, steps):
@@ -58,7 +58,7 @@ def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
     The reference asserts ndim >= 2 (muon.py:13) and normalises over the last two dimensions
     (muon.py:23), but its buffers and its symmetric kernel only admit 2-D input (muon.py:19-20,
     matmul_transpose_triton.py:83).  Here leading dimensions are a batch of independent matrices,
-    orthogonalised up to 16 per launch.
+    orthogonalised up to 32 per launch.
     """
     assert G.ndim >= 2
     assert G.is_cuda, "Input `d_in` must be a CUDA tensor"
@@ -95,7 +95,7 @@ class Muon(torch.optim.Optimizer):
         ns_steps: The number of Newton-Schulz iteration steps to use.
         rank, world_size: required, as in the reference; only (0, 1) is implemented.
         batch: (not in the reference) how many same-shape matrices are orthogonalised per launch,
-            1..16; default 16.
+            1..32; default 32.
 
     Not for embeddings, the final fully connected layer or 0/1-D parameters; 4-D convolution
     filters are flattened over their last three dimensions.

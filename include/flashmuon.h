@@ -181,7 +181,7 @@ FM_API int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int6
 FM_API size_t fm_newtonschulz_workspace_bytes(int rows, int cols);
 
 /* ---------------------------------------------------------------------------------------------
- * The same for `batch` (1..16) matrices of one shape and dtype, with every GEMM-shaped stage run
+ * The same for `batch` (1..32) matrices of one shape and dtype, with every GEMM-shaped stage run
  * as ONE launch over the whole batch, so that shapes whose tile count does not fill the chip
  * (M = 4096 gives 136 tiles for 256 CUs) are packed together.  G and out are HOST arrays of
  * `batch` device pointers; all inputs share ldg and all outputs ldout.  No out[i] may overlap
@@ -219,7 +219,7 @@ FM_API int fm_weight_update(void* p, int p_dtype, const void* u_bf16, int64_t n,
                      float alpha, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
- * The two updates above for `batch` (1..16) tensors of n elements each in one launch: g, buf, p and
+ * The two updates above for `batch` (1..32) tensors of n elements each in one launch: g, buf, p and
  * u_bf16 are HOST arrays of `batch` device pointers; tensor i gets exactly what the single-tensor
  * call computes.  No tensor may overlap another.  For the loop over same-shape parameters:
  * flash_muon/muon.py:90-100 and 86-89.
@@ -228,6 +228,18 @@ FM_API int fm_momentum_nesterov_batched(void* const* g, void* const* buf, int ba
                                  float w_buf, float w_nes, int nesterov, fm_stream_t stream);
 FM_API int fm_weight_update_batched(void* const* p, int p_dtype, const void* const* u_bf16, int batch,
                              int64_t n, float decay_mul, float alpha, fm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Measurement aid, no counterpart in the reference: `launches` launches of a kernel in which
+ * `blocks` workgroups of four waves each issue iters * 64 independent 32x32x16 bf16 MFMAs per wave on
+ * register operands taken from `operands` (blocks * 256 * 128 bytes: zeros, or N(0,1) bf16 values).
+ * After the last launch clocks[2*b] holds the shader cycles and clocks[2*b + 1] the 100 MHz
+ * real-time ticks workgroup b spent in its loop; sink takes blocks * 256 floats nobody needs.
+ * The flop count is blocks * 4 * iters * 64 * 32768 per launch.  bench.py --mfma-probe reports the
+ * sustained rate and clock with it: the ceiling the power cap sets for MFMA work on real data.
+ */
+FM_API int fm_probe_mfma_peak(const void* operands, int blocks, int iters, int launches, float* sink,
+                              long long* clocks, fm_stream_t stream);
 
 #ifdef __cplusplus
 }

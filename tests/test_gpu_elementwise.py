@@ -85,6 +85,6 @@ def test_batched_argument_errors(lib):
     b = torch.zeros(64, dtype=torch.bfloat16, device=DEV)
     s = gpu_util._stream(a)
     assert lib.fm_momentum_nesterov_batched(_ptrs([a, a]), _ptrs([b, b]), 2, 0, 64, 0.05, 0.95, 1, s) == 5   # same g twice
-    assert lib.fm_momentum_nesterov_batched(_ptrs([a]), _ptrs([b]), 17, 0, 64, 0.05, 0.95, 1, s) == 2       # batch > 16
+    assert lib.fm_momentum_nesterov_batched(_ptrs([a]), _ptrs([b]), 33, 0, 64, 0.05, 0.95, 1, s) == 2       # batch > 32
     assert lib.fm_weight_update_batched(_ptrs([a, b]), 0, _ptrs([b, a]), 2, 64, 1.0, 1.0, s) == 5            # p aliases u
     assert lib.fm_weight_update_batched(_ptrs([a]), 7, _ptrs([b]), 1, 64, 1.0, 1.0, s) == 4

@@ -131,7 +131,7 @@ def test_batched_matches_single_and_oracle(lib, rows, cols):
         # the batch changes which tiles fall into the split last round, hence fp32 summation order
         assert oracle.rel_fro(out, single.float()) < TOL
     # too many matrices, a missing pointer and an output aliasing another input are refused
-    assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 17)(), 0, 17, rows, cols, cols, (ctypes.c_void_p * 17)(), cols,
+    assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 33)(), 0, 33, rows, cols, cols, (ctypes.c_void_p * 33)(), cols,
                                             5, a, b, c, 1e-7, ws.data_ptr(), ws.numel(), None) == 2
     assert lib.fm_newtonschulz_batched_bf16((ctypes.c_void_p * 2)(Gs[0].data_ptr(), None), 0, 2, rows, cols, cols,
                                             (ctypes.c_void_p * 2)(outs[0].data_ptr(), outs[1].data_ptr()), cols,
@@ -143,9 +143,9 @@ def test_batched_matches_single_and_oracle(lib, rows, cols):
 
 def test_leading_dimensions_are_a_batch():
     """ndim > 2: every matrix of the leading dimensions is orthogonalised on its own (the norm of
-    muon.py:23 is over the last two dimensions), here 19 of them in chunks of 16 and 3."""
+    muon.py:23 is over the last two dimensions), here 35 of them in chunks of 32 and 3."""
     g = torch.Generator().manual_seed(31)
-    G = (1e-3 * torch.randn(19, 96, 160, generator=g)).bfloat16().to(DEV)
+    G = (1e-3 * torch.randn(35, 96, 160, generator=g)).bfloat16().to(DEV)
     out = fast_newtonschulz(G, 5)
     assert out.shape == G.shape and out.dtype == torch.bfloat16
     # against the CPU oracle on the whole batch (per-matrix norms, muon.py:23), every member
@@ -160,7 +160,7 @@ def test_leading_dimensions_are_a_batch():
     tall_got = fast_newtonschulz(Gc[:4].mT.contiguous().to(DEV), 5)
     assert tall_got.shape == (4, 160, 96)
     assert oracle.rel_fro(tall_got, tall_ref) < _tol(96, 160)
-    for i in (0, 7, 15, 16, 18):
+    for i in (0, 7, 31, 32, 34):
         assert torch.equal(out[i], fast_newtonschulz(G[i], 5))
     G4 = G[:6].reshape(2, 3, 96, 160)
     assert torch.equal(fast_newtonschulz(G4, 5), out[:6].reshape(2, 3, 96, 160))
