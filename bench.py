@@ -26,9 +26,9 @@ DIM = 8192
 # L2-miss traffic of one 8192^2 call (main kernel + the kernel that adds up the split last round),
 # from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
 # 128 MiB device copy (FETCH_SIZE reads half of the copied bytes there, WRITE_SIZE all of them):
-# (509.9e3 + 32.85e3) KiB * 2.0 fetched + (209.8e3 + 3.46e3) KiB written.  The commands and the raw
+# (505.6e3 + 32.85e3) KiB * 2.0 fetched + (210.1e3 + 3.46e3) KiB written.  The commands and the raw
 # readings are in profiles/syrk_bf16_8192_traffic.md.
-TRAFFIC_BYTES = int((509.9e3 + 32.85e3) * 1024 * 2.0 + (209.8e3 + 3.46e3) * 1024 * 1.0)
+TRAFFIC_BYTES = int((505.6e3 + 32.85e3) * 1024 * 2.0 + (210.1e3 + 3.46e3) * 1024 * 1.0)
 
 
 def _time_gpu(fn, steps, warmup, torch):
