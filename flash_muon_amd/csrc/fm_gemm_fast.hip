@@ -317,6 +317,9 @@ __device__ __forceinline__ void epilogue_quarter(const GemmArgs& g, bool diag, f
 // items left over are cut once more into `split` sub-parts each, one per workgroup, in a last round.
 // Anything that is not a whole tile is written to a partial-tile slot: item i of a full round to
 // slot i, sub-part q of left-over item j to slot tail_slot0 + j * split + q.
+// When whole tiles are left over and there are at most grid / 16 of them, the last round cuts them
+// in space instead (sub64): 16 sub-tiles of 64x64 per tile, one per workgroup, each over the whole
+// k, so that nothing has to be added up afterwards.
 struct FastArgs {
   GemmArgs g;
   float* partials;      // fp32 partial tiles
@@ -328,6 +331,7 @@ struct FastArgs {
   int split;            // sub-parts per item of the last round
   int tail_slot0;       // first slot of the last round's sub-parts
   int reduce_tile0;     // first tile the second kernel has to finish
+  int sub64;            // the left-over tiles are computed whole-k as 64x64 sub-tiles, 16 workgroups each
 };
 
 // k stages [kb, ke) of base part `part` of `parts`, or of its sub-part `sub` of `subs`
@@ -364,6 +368,145 @@ __device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& b, int&
     }
   }
   ti = tj = 0;   // not reached for pos < num_tiles
+}
+
+// ---- 64x64 sub-tiles of the tiles left over after the last full round ---------------------------
+// One workgroup per sub-tile, four waves of 32x32 (one MFMA tile each), the whole k range, so the
+// result needs no second pass and is summed in the same k order as a whole tile.  A sub-tile moves
+// four times the operand bytes per flop of a 256x256 tile and is bound by the copy path (16 KiB per
+// stage against 4 MFMAs per wave), hence a deep ring: 8 stages of 16 KiB, 7 in flight.
+constexpr int SUB = 64;
+constexpr int SUB_OPER = SUB * ROWB;          // 64 rows of one operand stage: 8 KiB
+constexpr int SUB_STAGE = 2 * SUB_OPER;
+constexpr int SUB_DEPTH = 8;
+constexpr int SUB_F_PITCH = 36;               // floats per staged column: 32 rows + 4 of padding
+
+template <bool F16>
+__device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, int si, int sj, int nk,
+                                           unsigned char* smem, int lane, int wave) {
+  const bool tdiag = g.symmetric && ti == tj;
+  if (tdiag && si > sj) return;               // the mirror image of sub-tile (sj, si) of the same tile
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = ti * BM + si * SUB, n0 = tj * BN + sj * SUB;
+
+  // copy q of this wave fills LDS rows wave*16 + q*8 .. +8 of an operand stage
+  uint32_t voA[2], voB[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int row = wave * 16 + q * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ swz(row);
+    voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
+    voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
+  }
+  const bf16_t* gA = g.A + (int64_t)m0 * g.lda;
+  const bf16_t* gB = g.B + (int64_t)n0 * g.ldb;
+  const uint32_t ldsw = FM_LDS_ADDR(smem) + wave * 2048;
+  auto issue = [&](int stage, int slot) {   // 4 copies per wave
+    const uint32_t base = ldsw + slot * SUB_STAGE;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) dma16(voA[q], gA + stage * BKF, base + q * 1024);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) dma16(voB[q], gB + stage * BKF, base + SUB_OPER + q * 1024);
+  };
+  uint32_t ao, bo;
+  {
+    const int ra = wm * 32 + (lane & 31), rb = wn * 32 + (lane & 31);
+    ao = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
+    bo = (uint32_t)(SUB_OPER + rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
+  }
+
+  f32x16_t acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  // stages past the end are the last stage again (into slots nobody reads), so that the number of
+  // copies in flight is the same at every wait
+#pragma unroll
+  for (int s = 0; s < SUB_DEPTH - 1; ++s) issue(s < nk ? s : nk - 1, s);
+  for (int s = 0; s < nk; ++s) {
+    wait_vmcnt<4 * (SUB_DEPTH - 2)>();   // my copies of stage s have landed ...
+    __syncthreads();                     // ... and everybody's; stage s-1 is read out everywhere
+    {
+      const int nx = s + SUB_DEPTH - 1;
+      issue(nx < nk ? nx : nk - 1, nx & (SUB_DEPTH - 1));
+    }
+    const unsigned char* st = smem + (s & (SUB_DEPTH - 1)) * SUB_STAGE;
+    bf16x8_t fa[4], fb[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      fa[ks] = *reinterpret_cast<const bf16x8_t*>(st + (ao ^ (ks << 5)));
+      fb[ks] = *reinterpret_cast<const bf16x8_t*>(st + (bo ^ (ks << 5)));
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) acc = mfma_32x32x16<F16>(fa[ks], fb[ks], acc);
+  }
+  wait_vmcnt<0>();
+  __syncthreads();   // no copy in flight and no wave still reading: the ring is free
+
+  // accumulators -> a wave-private staging block (column-major, 32 columns of 32 rows), then out:
+  // the direct pass writes 1 row x 16 columns per lane and puts the rounded values back, the
+  // transposed pass 16 rows x 1 column per lane, so both copies carry the same bits
+  float* const F = reinterpret_cast<float*>(smem + wave * (32 * SUB_F_PITCH * 4));
+  {
+    const int c = lane & 31, rg = 4 * (lane >> 5);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4_t v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+      *reinterpret_cast<f32x4_t*>(F + c * SUB_F_PITCH + 8 * q + rg) = v;
+    }
+  }
+  const int row0 = m0 + wm * 32, col0 = n0 + wn * 32;
+  // a block of a diagonal sub-tile holds its own mirror image (or is one of a pair of blocks that
+  // hold each other's, bit for bit): such a sub-tile is written once, by the direct pass
+  const bool bdiag = tdiag && si == sj;
+  const bool use_e = !F16 && g.E != nullptr;
+  const bool mirror = !bdiag && g.C2 != nullptr;
+  {
+    const int r = lane >> 1, c0 = (lane & 1) * 16;
+    const int row = row0 + r, col = col0 + c0;
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) v[k] = F[(c0 + k) * SUB_F_PITCH + r];
+    if (use_e) {
+      union { uint4 q[2]; unsigned short h[16]; } e;
+      const uint4* src = reinterpret_cast<const uint4*>(g.E + (int64_t)row * g.lde + col);
+      e.q[0] = src[0];
+      e.q[1] = src[1];
+      const float al = g.row_alpha ? g.alpha + g.row_alpha[row] : g.alpha;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) v[k] = __builtin_fmaf(al, elem_to_f32<F16>(e.h[k]), g.beta * v[k]);
+    }
+    if (bdiag && wm == wn && g.diag_out != nullptr) {   // this block lies on the diagonal of the product
+      const int kd = r - c0;                            // the diagonal element of this row, if 0..15
+      float dv = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const bool on = kd == k;
+        dv = on ? v[k] : dv;
+        v[k] = on ? 0.0f : v[k];
+      }
+      if ((unsigned)kd < 16u) g.diag_out[row] = dv;
+    }
+    union { uint4 q[2]; unsigned short h[16]; } o;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      o.h[k] = f32_to_elem<F16>(v[k]);
+      if (mirror) F[(c0 + k) * SUB_F_PITCH + r] = elem_to_f32<F16>(o.h[k]);
+    }
+    if (g.C) {
+      uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(g.C) + (int64_t)row * g.c_rs + col);
+      dst[0] = o.q[0];
+      dst[1] = o.q[1];
+    }
+  }
+  if (mirror) {
+    const int c = lane >> 1, r0 = (lane & 1) * 16;
+    union { uint4 q[2]; unsigned short h[16]; } o;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) o.h[k] = f32_to_elem<F16>(F[c * SUB_F_PITCH + r0 + k]);
+    uint4* dst = reinterpret_cast<uint4*>(reinterpret_cast<unsigned short*>(g.C2) + (int64_t)(col0 + c) * g.c2_rs + row0 + r0);
+    dst[0] = o.q[0];
+    dst[1] = o.q[1];
+  }
 }
 
 template <bool F16>
@@ -408,6 +551,13 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       item = round * p.grid + w;
       slot_id = item;
       item_range(p.nk, item % p.ksplit, p.ksplit, 0, 1, kb, ke);
+    } else if (p.sub64) {
+      if (w >= p.rem * 16) break;
+      int sbi, sti, stj;
+      tile_at(p.g, p.rounds * p.grid + (w >> 4), sbi, sti, stj);
+      const GemmArgs sg = batch_view(p.g, sbi);
+      sub64_tile<F16>(sg, sti, stj, (w >> 2) & 3, w & 3, p.nk, smem, lane, wave);
+      break;
     } else {
       if (w >= p.rem * p.split) break;
       const int j = w / p.split, sub = w - j * p.split;
@@ -767,6 +917,9 @@ static void fast_schedule(int num_tiles, int nk, long long max_slots, FastArgs& 
     if ((long long)f.rem * s > room) s = (int)(room / f.rem);
     f.split = s < 1 ? 1 : s;
   }
+  // whole tiles left over, few enough for 16 workgroups each: cut them in space, not along k
+  f.sub64 = (ksplit == 1 && f.rem > 0 && f.rem * 16 <= grid && knob(kKnobNoSub64) <= 0) ? 1 : 0;
+  if (f.sub64) f.split = 1;
   f.tail_slot0 = ksplit > 1 ? f.rounds * grid : 0;
   // whole tiles need no second kernel: with ksplit == 1 only the left-over items, if they were cut
   f.reduce_tile0 = ksplit > 1 ? 0 : (f.split > 1 ? f.rounds * grid : num_tiles);

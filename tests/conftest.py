@@ -22,7 +22,8 @@ def lib():
     return _lib.load()
 
 
-KNOBS = {"FLASHMUON_GRID": 0, "FLASHMUON_KSPLIT": 1, "FLASHMUON_FAST_MIN_UNITS": 2, "FLASHMUON_NO_MID": 3}
+KNOBS = {"FLASHMUON_GRID": 0, "FLASHMUON_KSPLIT": 1, "FLASHMUON_FAST_MIN_UNITS": 2, "FLASHMUON_NO_MID": 3,
+         "FLASHMUON_NO_SUB64": 4}
 
 
 @pytest.fixture

@@ -154,3 +154,78 @@ def test_fast_and_general_paths_agree_on_gaussian_input(lib):
     for Y in (fast, slow):
         assert float((Y.float() - ref).norm() / ref.norm()) < 3e-3
     assert torch.equal(matmul_transpose(X), fast)
+
+
+@pytest.mark.parametrize("no_sub64", [0, 1])
+@pytest.mark.parametrize("M,K,grid", [(2048, 1024, 34), (2048, 320, 35), (1536, 2048, 20), (2304, 512, 43), (2048, 64, 34)])
+def test_syrk_fast_last_round_in_space_or_along_k(lib, knobs, M, K, grid, no_sub64):
+    """One or two whole tiles left after the last full round (the GRID knob makes small inputs end
+    that way; at 8192^2 on 256 CUs it is 16 of 528): by default they are computed as 64x64
+    sub-tiles over the whole k, 16 workgroups each, with NO_SUB64 they are cut along k into fp32
+    parts and added up by the second kernel.  The left-over tiles include a diagonal one (written
+    once) and an off-diagonal one (written twice)."""
+    knobs("FLASHMUON_GRID", grid)
+    knobs("FLASHMUON_NO_SUB64", no_sub64)
+    X = _ints((M, K), M + 3 * K + grid)
+    want = _exact(X.double() @ X.double().T)
+    Y = torch.full((M, M), 7.0, dtype=torch.bfloat16, device=DEV)
+    if no_sub64:
+        gpu_util.syrk(lib, X.to(DEV), Y)
+    else:                                              # the cut in space needs no workspace at all
+        Xd = X.to(DEV)
+        st = lib.fm_syrk_bf16(Xd.data_ptr(), K, Y.data_ptr(), M, 1, M, K, None, 0, gpu_util._stream(Xd))
+        assert st == 0
+    assert torch.equal(Y.cpu(), want)
+    assert torch.equal(Y, Y.T)
+    # Gaussian input: both ways of cutting sum every element in the same k order as a whole tile
+    g = torch.Generator().manual_seed(grid)
+    G = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    got = gpu_util.syrk(lib, G)
+    assert torch.equal(got, got.T)
+    knobs("FLASHMUON_GRID", -1)
+    knobs("FLASHMUON_NO_SUB64", -1)
+    whole = gpu_util.syrk(lib, G)                      # every tile whole (no left-over at this size on 256 CUs)
+    if not no_sub64:
+        assert torch.equal(got, whole)
+    else:
+        assert float((got.float() - whole.float()).norm() / whole.float().norm()) < 1e-3
+
+
+@pytest.mark.parametrize("no_sub64", [0, 1])
+def test_poly_and_axpby_fast_last_round_in_space(lib, knobs, no_sub64):
+    """The epilogue operand, the fp32 diagonal and the per-row addition on the 64x64 sub-tiles."""
+    knobs("FLASHMUON_NO_SUB64", no_sub64)
+    knobs("FLASHMUON_GRID", 34)
+    M = 2048
+    g = torch.Generator().manual_seed(9)
+    A = torch.randint(-1, 2, (M, M), generator=g)
+    A = (torch.triu(A) + torch.triu(A, 1).T).float().bfloat16()
+    Ad = A.double()
+    full = Ad + 2 * (Ad @ Ad)
+    assert torch.equal(gpu_util.syrk_poly(lib, A.to(DEV), 1.0, 2.0).cpu(), _exact(full))
+    P, d = gpu_util.syrk_poly(lib, A.to(DEV), 1.0, 2.0, split_diag=True)
+    assert torch.equal(d.cpu().double(), torch.diagonal(full))
+    assert torch.equal(P.cpu(), _exact(full - torch.diag(torch.diagonal(full))))
+    assert torch.equal(P, P.T)
+    knobs("FLASHMUON_GRID", 17)                        # 3 x 6 = 18 tiles: one left over
+    M, K = 768, 1536
+    Pm = _ints((M, M), 31, -1, 1)
+    X = _ints((M, K), 37)
+    dd = torch.arange(M, dtype=torch.float32) % 3 - 1
+    want = _exact((2 + dd.double())[:, None] * X.double() + Pm.double() @ X.double())
+    Xo, XoT = gpu_util.gemm_axpby(lib, Pm.to(DEV), X.to(DEV), 2.0, row_alpha=dd.to(DEV))
+    assert torch.equal(Xo.cpu(), want)
+    assert torch.equal(XoT.cpu(), want.T)
+    only_t = gpu_util.gemm_axpby(lib, Pm.to(DEV), X.to(DEV), 2.0, want_x=False, row_alpha=dd.to(DEV))[1]
+    assert torch.equal(only_t.cpu(), want.T)
+
+
+def test_syrk_f16_fast_last_round_in_space(lib, knobs):
+    knobs("FLASHMUON_GRID", 34)
+    X = _ints((2048, 512), 5).half()
+    want = (X.double() @ X.double().T).half()
+    Xd = X.to(DEV)
+    Y = torch.full((2048, 2048), 7.0, dtype=torch.float16, device=DEV)
+    st = lib.fm_syrk_f16(Xd.data_ptr(), 512, Y.data_ptr(), 2048, 1, 2048, 512, None, 0, gpu_util._stream(Xd))
+    assert st == 0
+    assert torch.equal(Y.cpu(), want)
