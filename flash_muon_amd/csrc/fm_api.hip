@@ -175,7 +175,7 @@ int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, int M, f
                    overlaps(mat_range(diag_out, 1, M, M, 4), mat_range(P, M, M, ldp, 2))))
     return FM_ERR_ALIAS;
   GemmArgs a = {};
-  a.A = a.B = a.E = static_cast<const bf16_t*>(A); a.lda = a.ldb = a.lde = lda;
+  a.A = a.B = a.E = a.ET = static_cast<const bf16_t*>(A); a.lda = a.ldb = a.lde = a.ldet = lda;   // A is symmetric
   a.C = a.C2 = static_cast<bf16_t*>(P);
   a.c_rs = a.c2_rs = ldp; a.c_cs = a.c2_cs = 1;
   a.Ma = a.Nb = a.Kc = M;
@@ -209,6 +209,7 @@ int fm_gemm_axpby_bf16(const void* P, int64_t ldp, const void* XT, int64_t ldxt,
   a.A = static_cast<const bf16_t*>(P); a.lda = ldp;
   a.B = static_cast<const bf16_t*>(XT); a.ldb = ldxt;
   a.E = static_cast<const bf16_t*>(X); a.lde = ldx;
+  a.ET = a.B; a.ldet = ldxt;
   a.C = static_cast<bf16_t*>(Xout); a.c_rs = ldo; a.c_cs = 1;
   a.C2 = static_cast<bf16_t*>(XoutT); a.c2_rs = ldot; a.c2_cs = 1;
   a.Ma = M; a.Nb = K; a.Kc = M;
@@ -338,8 +339,8 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
     if (launch_gemm_nt(g, gws, gws_bytes, hs)) return FM_ERR_LAUNCH;
     // P = b A + c A A, diagonal in fp32
     g = GemmArgs{};
-    g.A = g.B = g.E = A; g.lda = g.ldb = g.lde = M;
-    g.bs_a = g.bs_b = g.bs_e = mm;
+    g.A = g.B = g.E = g.ET = A; g.lda = g.ldb = g.lde = g.ldet = M;
+    g.bs_a = g.bs_b = g.bs_e = g.bs_et = mm;
     g.C = g.C2 = P; g.c_rs = g.c2_rs = M; g.c_cs = g.c2_cs = 1; g.bs_c = g.bs_c2 = mm;
     g.Ma = g.Nb = g.Kc = M; g.alpha = b; g.beta = c; g.symmetric = 1; g.batch = batch;
     g.diag_out = pdiag; g.bs_do = (int64_t)l.pdiag_stride;
@@ -349,6 +350,7 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
     g.A = P; g.lda = M; g.bs_a = mm;
     g.B = XT; g.ldb = M; g.bs_b = mk;
     g.E = X; g.lde = K; g.bs_e = mk;
+    g.ET = XT; g.ldet = M; g.bs_et = mk;
     g.Ma = M; g.Nb = K; g.Kc = M; g.alpha = a; g.beta = 1.0f; g.symmetric = 0; g.batch = batch;
     g.row_alpha = pdiag; g.bs_ra = (int64_t)l.pdiag_stride;
     g.c_cs = g.c2_cs = 1;

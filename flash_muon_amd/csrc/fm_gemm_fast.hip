@@ -9,6 +9,8 @@
 // part per workgroup, so that the last round is as short as its share of the work; the parts go to
 // memory as fp32 and a second, small kernel adds them in part order and runs the epilogue.
 #include "fm_internal.h"
+
+#include <type_traits>
 #include <cstdlib>
 
 namespace fm {
@@ -173,12 +175,16 @@ template <int I, int NI>
 __device__ __forceinline__ void stage_store(const f32x16_t (&acc)[NI][4], float* F, int lane) {
   const int c = lane & 31, rg = 4 * (lane >> 5);
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      f32x4_t v = {acc[I][j][4 * q], acc[I][j][4 * q + 1], acc[I][j][4 * q + 2], acc[I][j][4 * q + 3]};
-      *reinterpret_cast<f32x4_t*>(F + qf_idx(32 * j + c, 8 * q + rg)) = v;
-    }
+  for (int j = 0; j < 4; ++j) {
+    // (sub-vectors, not element reads: see the note on identical element reads at epilogue_regs)
+    const f32x16_t a = acc[I][j];
+    float* const dst = F + (32 * j + c) * QF_PITCH;
+    const int x = ((32 * j + c) >> 3 & 7) << 2;
+    *reinterpret_cast<f32x4_t*>(dst + ((0 + rg) ^ x)) = __builtin_shufflevector(a, a, 0, 1, 2, 3);
+    *reinterpret_cast<f32x4_t*>(dst + ((8 + rg) ^ x)) = __builtin_shufflevector(a, a, 4, 5, 6, 7);
+    *reinterpret_cast<f32x4_t*>(dst + ((16 + rg) ^ x)) = __builtin_shufflevector(a, a, 8, 9, 10, 11);
+    *reinterpret_cast<f32x4_t*>(dst + ((24 + rg) ^ x)) = __builtin_shufflevector(a, a, 12, 13, 14, 15);
+  }
 }
 
 // the 128 x 32 floats of the staged quarter, in staging order, to a partial-tile slot (coalesced)
@@ -235,14 +241,54 @@ __device__ __forceinline__ void epi_dma_e(const GemmArgs& g, int row_base, int c
 // x_ik * x_jk in the same order, through the same dot-product datapath.  So such a tile is written
 // once, whole, by the direct pass and has no transposed pass.  The fp32 diagonal, if asked for, is
 // split off here.
+// G iterations of the direct pass with an operand E, off the diagonal: every LDS read of the batch
+// is issued before the first value is put back into F, so the batch pays one LDS round trip and
+// not one per iteration (a read may not be moved above an earlier write to F by the compiler).
+template <bool F16, int G>
+__device__ __forceinline__ void direct_e_batch(const GemmArgs& g, float* F, const unsigned char* Eb, const float* RA,
+                                               int ra_off, int row_base, int col_base, int lane, int it0) {
+  const float alpha = g.alpha, beta = g.beta;
+  unsigned short* C = reinterpret_cast<unsigned short*>(g.C);
+  float v[G][8], al[G];
+  union { uint4 v; unsigned short s[8]; } e[G];
+#pragma unroll
+  for (int n = 0; n < G; ++n) {
+    const int idx = (it0 + n) * 64 + lane;
+    const int r = idx >> 4, c0 = (idx & 15) * 8;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[n][k] = F[qf_idx(c0 + k, r)];
+    e[n].v = *reinterpret_cast<const uint4*>(Eb + r * 256 + c0 * 2);
+    al[n] = alpha + RA[ra_off + r];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int n = 0; n < G; ++n) {
+    const int idx = (it0 + n) * 64 + lane;
+    const int r = idx >> 4, c0 = (idx & 15) * 8;
+    union { uint4 v; unsigned short s[8]; } o;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      o.s[k] = f32_to_elem<F16>(__builtin_fmaf(al[n], elem_to_f32<F16>(e[n].s[k]), beta * v[n][k]));
+      F[qf_idx(c0 + k, r)] = elem_to_f32<F16>(o.s[k]);   // what the transposed pass stores
+    }
+    if (C) *reinterpret_cast<uint4*>(C + (int64_t)(row_base + r) * g.c_rs + col_base + c0) = o.v;
+  }
+}
+
 template <bool F16, bool HAS_E, bool DIAG>
 __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, const unsigned char* Eb,
                                                    const float* RA, int ra_off, int row_base, int col_base,
                                                    int lane, int it_begin, int it_end, int passes) {
   const float alpha = g.alpha, beta = g.beta;
   const bool dout = DIAG && g.diag_out != nullptr;
-  const bool has_ra = HAS_E && g.row_alpha != nullptr;
-  if ((passes & 1) && (g.C || HAS_E)) {
+  if constexpr (HAS_E && !DIAG) {
+    if (passes & 1) {
+      int it = it_begin;
+      for (; it + 4 <= it_end; it += 4) direct_e_batch<F16, 4>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it);
+      for (; it + 2 <= it_end; it += 2) direct_e_batch<F16, 2>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it);
+      if (it < it_end) direct_e_batch<F16, 1>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it);
+    }
+  } else if ((passes & 1) && (g.C || HAS_E)) {
     unsigned short* C = reinterpret_cast<unsigned short*>(g.C);
 #pragma unroll 4
     for (int it = it_begin; it < it_end; ++it) {
@@ -255,7 +301,7 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
       union { uint4 v; unsigned short s[8]; } e, o;
       if (HAS_E) {
         e.v = *reinterpret_cast<const uint4*>(Eb + r * 256 + c0 * 2);
-        const float al = has_ra ? alpha + RA[ra_off + r] : alpha;
+        const float al = alpha + RA[ra_off + r];
 #pragma unroll
         for (int k = 0; k < 8; ++k) v[k] = __builtin_fmaf(al, elem_to_f32<F16>(e.s[k]), beta * v[k]);
       }
@@ -271,10 +317,7 @@ __device__ __forceinline__ void epilogue_quarter_t(const GemmArgs& g, float* F, 
         if (dout && (unsigned)kd < 8u) g.diag_out[row] = dv;
       }
 #pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        o.s[k] = f32_to_elem<F16>(v[k]);
-        if (HAS_E && !DIAG) F[qf_idx(c0 + k, r)] = elem_to_f32<F16>(o.s[k]);   // what the transposed pass stores
-      }
+      for (int k = 0; k < 8; ++k) o.s[k] = f32_to_elem<F16>(v[k]);
       if (g.C) *reinterpret_cast<uint4*>(C + (int64_t)row * g.c_rs + col) = o.v;
     }
   }
@@ -309,6 +352,218 @@ __device__ __forceinline__ void epilogue_quarter(const GemmArgs& g, bool diag, f
   }
   if (diag) epilogue_quarter_t<F16, false, true>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
   else epilogue_quarter_t<F16, false, false>(g, F, Eb, RA, ra_off, row_base, col_base, lane, it_begin, it_end, passes);
+}
+
+// ---- write-out of a whole tile from the accumulators --------------------------------------------
+// An MFMA accumulator register pair of a lane holds two consecutive rows of one column, which is
+// what the transposed output wants: after rounding, the pairs go to C2 straight from the
+// registers (two lanes 32 apart swap halves first, so that every lane stores 8 consecutive rows,
+// 16 bytes).  Only the direct output needs the transposition through LDS, and it stages the rounded
+// 16-bit values: neighbouring lanes (columns c and c+1) exchange halves, so that every lane holds
+// two consecutive columns of one row, and a quarter (32 rows x 128 columns) is staged row-major,
+// 8 KiB instead of 16 KiB of fp32, and read back 16 bytes per lane.  Both copies carry the same bits.
+// The operand E is read transposed (ET) in the accumulators' own layout, 8 consecutive rows of one
+// column per lane and load, so the arithmetic happens in registers before anything is staged.
+constexpr int QT_PITCH = 320;             // bytes per staged row: 128 values + 64 bytes, so that rows r and r+1 use different banks
+constexpr int QT_BYTES = 32 * QT_PITCH;   // one staged quarter of a wave
+constexpr int QS_OFFSET = QT_BYTES + 512; // after it the row additions, then the quarter's accumulators (16 KiB)
+static_assert(QS_OFFSET + 16 * 1024 <= EPI_WAVE_BYTES, "the write-out stages inside the wave's region");
+
+// 16 bytes per lane at base + voff + soff (bytes) through a buffer descriptor: the per-lane part of
+// an address is one 32-bit register, the rest is scalar
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t block_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+}
+__device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t b, uint32_t voff, int soff) {
+  const v4i_t v = __builtin_amdgcn_raw_buffer_load_b128(b, (int)voff, soff, 0);
+  return uint4{(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
+}
+__device__ __forceinline__ void buf_store16(__amdgpu_buffer_rsrc_t b, uint32_t voff, int soff, const uint4& d) {
+  const v4i_t v = {(int)d.x, (int)d.y, (int)d.z, (int)d.w};
+  __builtin_amdgcn_raw_buffer_store_b128(v, b, (int)voff, soff, 0);
+}
+
+// One accumulator element, copied out of the accumulator file at this point of the program: left
+// to the compiler, all 256 are copied where the main loop ends, and do not fit.
+__device__ __forceinline__ float acc_read(float a) {
+  float v;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
+  return v;
+}
+
+__device__ __forceinline__ void swap32(uint32_t& lo_half_keeps, uint32_t& hi_half_keeps) {
+  // lanes 0..31 give `hi_half_keeps` to, and take `lo_half_keeps` of, the lane 32 above
+  const auto r = __builtin_amdgcn_permlane32_swap(lo_half_keeps, hi_half_keeps, false, false);
+  lo_half_keeps = r[0];
+  hi_half_keeps = r[1];
+}
+
+// two values rounded to the element type, `lo` in the low half
+template <bool F16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  if constexpr (F16) {
+    typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2_t));
+  } else {
+    typedef __bf16 b2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, b2_t));
+  }
+}
+
+// MODE: 0 without the operand E, 1 with it and beta == 1 (the product is added as it is), 2 with it
+// and any beta.  A kernel holds one instance only: of identical element reads in several branches
+// the optimizer makes one read of all 256 accumulators ahead of the branch, and they do not fit
+// into the vector registers.
+template <bool F16, int MODE>
+__device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool diag_block,
+                                              const f32x16_t (&acc)[4][4], unsigned char* T, int row0, int col0,
+                                              int lane) {
+  // what follows is derived from `lane` anew for every tile: kept in registers across the main
+  // loop instead, the per-lane offsets of the write-out would crowd out the loop's own
+  asm volatile("" : "+v"(lane));
+  constexpr bool has_e = !F16 && MODE != 0;
+  const int lc = lane & 31, lh = lane >> 5, par = lane & 1;
+  const bool direct = g.C != nullptr;
+  const bool mirror = g.C2 != nullptr && !diag;
+  const bool dout = diag && diag_block && g.diag_out != nullptr;
+  const float alpha = g.alpha, beta = g.beta;
+  const uint32_t sel = par ? 0x03020706u : 0x05040100u;   // odd lanes keep the high halves, even lanes the low ones
+  float* const RA = reinterpret_cast<float*>(T + QT_BYTES);
+  // staging: this lane writes row 8qq + 4lh + 2h + par, columns 32j + (lc & ~1) .. +1, and reads
+  // row 4it + lane/16, columns 8(lane % 16) .. +7
+  unsigned char* const tw = T + (4 * lh + par) * QT_PITCH + (lc & ~1) * 2;
+  const unsigned char* const tr = T + (lane >> 4) * QT_PITCH + (lane & 15) * 16;
+  // Global accesses go through buffer descriptors based at the wave's block, so that an address is
+  // one of three per-lane byte offsets plus a scalar offset:
+  // rows 32i + 16t + 8lh .. +7 of column 32j + lc are what a lane loads of ET and stores to C2,
+  // row 4it + lane/16, columns 8(lane % 16) .. +7 what it stores to C.
+  const uint32_t et_lane = (uint32_t)(lc * (int)g.ldet + 8 * lh) * 2u;
+  const uint32_t c2_lane = (uint32_t)(lc * (int)g.c2_rs + 8 * lh) * 2u;
+  const uint32_t c_lane = (uint32_t)((lane >> 4) * (int)g.c_rs + (lane & 15) * 8) * 2u;
+  const __amdgpu_buffer_rsrc_t et_buf = block_rsrc(g.ET + (int64_t)col0 * g.ldet + row0);
+  const __amdgpu_buffer_rsrc_t c2_buf = block_rsrc(g.C2 + (int64_t)col0 * g.c2_rs + row0);
+  const __amdgpu_buffer_rsrc_t c_buf = block_rsrc(g.C + (int64_t)row0 * g.c_rs + col0);
+  const int et_col = 64 * (int)g.ldet, c2_col = 64 * (int)g.c2_rs, c_row = 8 * (int)g.c_rs;   // bytes: 32 columns, 32 columns, 4 rows
+#define FM_ET(i, j, t) buf_load16(et_buf, et_lane, (j) * et_col + 64 * (i) + 32 * (t))
+
+  uint4 ev[4][2];
+  if constexpr (has_e) {
+    // the block's 128 additions to alpha (zeros when there are none), before any store of this tile
+    float2 ra = {0.0f, 0.0f};
+    if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+    *reinterpret_cast<float2*>(RA + lane * 2) = ra;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) ev[j][t] = FM_ET(0, j, t);
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f32x4_t al[4];
+    if constexpr (has_e) {
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq) {
+        al[qq] = *reinterpret_cast<const f32x4_t*>(RA + 32 * i + 8 * qq + 4 * lh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) al[qq][e] += alpha;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      // the scheduler works on one MFMA tile at a time: left alone with the whole unrolled
+      // write-out, it moves every accumulator to a vector register first and runs out of them
+      __builtin_amdgcn_sched_barrier(0);
+      // DOUT: the fp32 diagonal is split off and stored as zero.  A variant of the whole body, not
+      // a branch inside it, which would make the sixteen values a merge of two vectors.
+      auto tile = [&](auto dout_tag) {
+      constexpr bool DOUT = decltype(dout_tag)::value;
+      float v[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) v[r] = acc[i][j][r];
+      if constexpr (has_e) {
+        uint32_t eb[4][2];   // [qq][h]: the operand in the accumulators' layout
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          uint32_t a0 = ev[j][t].x, a1 = ev[j][t].y, b0 = ev[j][t].z, b1 = ev[j][t].w;
+          swap32(a0, b0);
+          swap32(a1, b1);
+          eb[2 * t][0] = a0; eb[2 * t][1] = a1; eb[2 * t + 1][0] = b0; eb[2 * t + 1][1] = b1;
+          if (i < 3) ev[j][t] = FM_ET(i + 1, j, t);
+        }
+        if constexpr (MODE == 2) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) v[r] *= beta;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const uint32_t w = eb[r >> 2][(r >> 1) & 1];
+          const float ef = elem_to_f32<F16>((unsigned short)((r & 1) ? (w >> 16) : (w & 0xffffu)));
+          v[r] = __builtin_fmaf(al[r >> 2][r & 3], ef, v[r]);
+        }
+      }
+      if constexpr (DOUT) {
+        float dv = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const bool on = lc == 8 * (r >> 2) + 4 * lh + (r & 3);
+          dv = on ? v[r] : dv;
+          v[r] = on ? 0.0f : v[r];
+        }
+        if (lh == ((lc >> 2) & 1)) g.diag_out[row0 + 32 * i + lc] = dv;
+      }
+      uint32_t P[4][2];   // [qq][h]: rows 8qq + 4lh + 2h, +1 of column 32j + lc, rounded
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) P[qq][h] = pack2<F16>(v[4 * qq + 2 * h], v[4 * qq + 2 * h + 1]);
+      if (direct) {   // stage the column of the quarter for the direct output
+#pragma unroll
+        for (int qq = 0; qq < 4; ++qq)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const uint32_t own = P[qq][h];
+            const uint32_t nbr = __builtin_amdgcn_update_dpp(0u, own, 0xB1, 0xF, 0xF, true);   // lane ^ 1
+            *reinterpret_cast<uint32_t*>(tw + (8 * qq + 2 * h) * QT_PITCH + 64 * j) = __builtin_amdgcn_perm(nbr, own, sel);
+          }
+      }
+      if (mirror) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          uint4 o = {P[2 * t][0], P[2 * t][1], P[2 * t + 1][0], P[2 * t + 1][1]};
+          swap32(o.x, o.z);   // now rows 16t + 8lh .. +7, in the order x y z w
+          swap32(o.y, o.w);
+          buf_store16(c2_buf, c2_lane, j * c2_col + 64 * i + 32 * t, o);
+        }
+      }
+      };
+      if (i == j && dout) tile(std::true_type{});
+      else tile(std::false_type{});
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // Every load of the tile has arrived long ago.  Said once in a form the compiler's bookkeeping
+    // of outstanding loads understands: it does not see the waits written in assembly, takes some
+    // load for pending when the next tile begins, and waits for everything in flight in the middle
+    // of the main loop.
+    if constexpr (has_e) {
+      if (i == 3) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    }
+
+    if (direct) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint4 d[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) d[it] = *reinterpret_cast<const uint4*>(tr + 4 * (4 * half + it) * QT_PITCH);
+#pragma unroll
+        for (int it = 0; it < 4; ++it) buf_store16(c_buf, c_lane, (8 * i + 4 * half + it) * c_row, d[it]);
+      }
+    }
+  }
+#undef FM_ET
 }
 
 // The schedule works on items: item i is base part i % ksplit of tile i / ksplit, where every tile's
@@ -509,7 +764,8 @@ __device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, in
   }
 }
 
-template <bool F16>
+// MODE: how whole tiles are written out (see epilogue_regs); chosen by the host from E and beta
+template <bool F16, int MODE>
 __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // two operand stages (A0 B0 A1 B1, 32 KiB each) during the main loop, the accumulator staging of
   // the four waves afterwards
@@ -645,47 +901,29 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
     }
 
-    // ---- accumulators -> LDS a quarter at a time, and out (see the notes above EpiLds) -----------
+    // ---- write-out -------------------------------------------------------------------------------
     const bool split = (n != p.nk);
     const bool diag = g.symmetric && ti == tj;
-    const EpiLds L = epi_lds(smem + wave * EPI_WAVE_BYTES);
-    float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
     const int row0 = m0 + wm * 128, col0 = n0 + wn * 128;
-    const bool use_e = !F16 && !split && g.E != nullptr;
-    if (use_e) {
-      epi_dma_e(g, row0, col0, lane, L.e_addr[0], 0, 8);
-      if (g.row_alpha) {   // the block's 128 rows, before any store of this tile
-        const float2 ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
-        *reinterpret_cast<float2*>(L.RA + lane * 2) = ra;
-      }
-    }
-    // The wait for quarter q's operand must not wait for the stores of quarter q-1, which were
-    // issued after its copies: it allows as many operations in flight as are known to follow them
-    // (8 copies of the next operand, 8 stores per output written; a diagonal tile writes one output,
-    // and the stores of its fp32 diagonal only make the wait longer than it has to be).
-#define FM_QUARTER(q)                                                                                  \
-    {                                                                                                  \
-      if (use_e && q < 3) epi_dma_e(g, row0 + 32 * (q + 1), col0, lane, L.e_addr[(q + 1) & 1], 0, 8);  \
-      stage_store<q, 4>(acc, L.F, lane);                                                                  \
-      if (split) {                                                                                     \
-        copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);                           \
-      } else {                                                                       \
-        if (use_e) {                                                                                   \
-          const int later = (q < 3 ? 8 : 0);                                                           \
-          const int stores = q == 0 ? 0 : ((g.C ? 8 : 0) + (g.C2 && !diag ? 8 : 0));                  \
-          if (later + stores >= 24) wait_vmcnt<24>();                                                  \
-          else if (later + stores >= 16) wait_vmcnt<16>();                                             \
-          else if (later + stores >= 8) wait_vmcnt<8>();                                               \
-          else wait_vmcnt<0>();                                                                        \
-        }                                                                                              \
-        epilogue_quarter<F16>(g, diag, L.F, L.E[q & 1], L.RA, 32 * q, row0 + 32 * q, col0, lane, 0, 8, 3);  \
-      }                                                                                                \
-    }
-    FM_QUARTER(0)
-    FM_QUARTER(1)
-    FM_QUARTER(2)
-    FM_QUARTER(3)
+    unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
+    if (split) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
+      const EpiLds L = epi_lds(wave_lds);
+      float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
+#define FM_QUARTER(q)                                                        \
+      stage_store<q, 4>(acc, L.F, lane);                                     \
+      copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);
+      FM_QUARTER(0)
+      FM_QUARTER(1)
+      FM_QUARTER(2)
+      FM_QUARTER(3)
 #undef FM_QUARTER
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));
+      epilogue_regs<F16, MODE>(g, diag, wm == wn, acc, wave_lds, row0, col0, lane);
+    }
     __syncthreads();   // the next tile's copies land in the memory the staging just used
   }
 }
@@ -708,8 +946,9 @@ __global__ __launch_bounds__(256) void gemm_nt_reduce_kernel(FastArgs p) {
   const int row0 = ti * BM + (blk >> 1) * 128, col0 = tj * BN + (blk & 1) * 128;
   if (g.E) {
     epi_dma_e(g, row0 + 32 * q, col0, lane, L.e_addr[0], wave * 2, wave * 2 + 2);
-    if (g.row_alpha && wave == 0) {
-      const float2 ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+    if (wave == 0) {
+      float2 ra = {0.0f, 0.0f};
+      if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
       *reinterpret_cast<float2*>(L.RA + lane * 2) = ra;
     }
   }
@@ -863,7 +1102,7 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
   // one quarter per wave: accumulators -> LDS, then out (the staging areas lie in the ring)
   float* const F = reinterpret_cast<float*>(smem + wave * (QF_FLOATS * 4));
   float* const RA = reinterpret_cast<float*>(smem + 4 * (QF_FLOATS * 4) + wave * 128);
-  if (use_e && g.row_alpha && lane < 32) RA[lane] = ra;
+  if (use_e && lane < 32) RA[lane] = ra;   // zeros when there are no per-row additions
   stage_store<0, 1>(acc, F, lane);
   const bool diag = g.symmetric && ti == tj;
   epilogue_quarter<F16>(g, diag, F, e_buf, RA, 0, row0, col0, lane, 0, 8, 3);
@@ -935,8 +1174,8 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
   if (a.Ma % tile != 0 || a.Nb % tile != 0) return false;       // whole tiles only: no edge masks here
   // in-tile byte offsets stay below 2^31
   if (a.lda >= (1 << 21) || a.ldb >= (1 << 21)) return false;
-  if (a.C && a.c_cs != 1) return false;
-  if (a.C2 && a.c2_cs != 1) return false;
+  if (a.C && (a.c_cs != 1 || a.c_rs >= (1 << 21))) return false;
+  if (a.C2 && (a.c2_cs != 1 || a.c2_rs >= (1 << 21))) return false;
   // 16-byte accesses of the epilogue
   if (a.C && (a.c_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C) & 15))) return false;
   if (a.C2 && (a.c2_rs % 8 != 0 || (reinterpret_cast<uintptr_t>(a.C2) & 15))) return false;
@@ -952,6 +1191,8 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
 
 bool gemm_fast_eligible(const GemmArgs& a) {
   if (!tiled_dma_eligible(a, BM)) return false;
+  // the write-out reads the epilogue operand transposed, 16 bytes at a time
+  if (a.E && (!a.ET || a.ldet % 8 != 0 || a.ldet >= (1 << 21) || (reinterpret_cast<uintptr_t>(a.ET) & 15) || (a.batch > 1 && a.bs_et % 8))) return false;
   const long long tm = a.Ma / BM, tn = a.Nb / BN;
   const long long tiles = (a.symmetric ? tm * (tm + 1) / 2 : tm * tn) * (a.batch < 1 ? 1 : a.batch);
   const int nk = a.Kc / BKF;
@@ -1019,11 +1260,13 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   const int reduce_tiles = a.num_tiles - f.reduce_tile0;
   if (reduce_tiles > 0 && (slots > have || f.ksplit * f.split > kMaxParts)) return kErrWorkspace;
   if (a.elem == kElemF16) {
-    hipLaunchKernelGGL(gemm_nt_rounds_kernel<true>, dim3(f.grid), dim3(256), 0, stream, f);
+    hipLaunchKernelGGL((gemm_nt_rounds_kernel<true, 0>), dim3(f.grid), dim3(256), 0, stream, f);
     if (reduce_tiles > 0)
       hipLaunchKernelGGL(gemm_nt_reduce_kernel<true>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
   } else {
-    hipLaunchKernelGGL(gemm_nt_rounds_kernel<false>, dim3(f.grid), dim3(256), 0, stream, f);
+    if (!a.E) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 0>), dim3(f.grid), dim3(256), 0, stream, f);
+    else if (a.beta == 1.0f) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 1>), dim3(f.grid), dim3(256), 0, stream, f);
+    else hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 2>), dim3(f.grid), dim3(256), 0, stream, f);
     if (reduce_tiles > 0)
       hipLaunchKernelGGL(gemm_nt_reduce_kernel<false>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
   }

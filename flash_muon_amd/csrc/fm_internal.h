@@ -78,6 +78,7 @@ struct GemmArgs {
   const bf16_t* A;  int64_t lda;
   const bf16_t* B;  int64_t ldb;
   const bf16_t* E;  int64_t lde;
+  const bf16_t* ET; int64_t ldet;   // E transposed (Nb x Ma), optional: the 256x256 path reads the operand through it
   bf16_t* C;  int64_t c_rs, c_cs;
   bf16_t* C2; int64_t c2_rs, c2_cs;
   int Ma, Nb, Kc;
@@ -89,7 +90,7 @@ struct GemmArgs {
   // `batch` independent problems of the same shape in one launch: matrix b of an operand starts
   // b * stride elements after matrix 0 (strides of absent operands are ignored)
   int batch;
-  int64_t bs_a, bs_b, bs_e, bs_c, bs_c2, bs_ra, bs_do;
+  int64_t bs_a, bs_b, bs_e, bs_et, bs_c, bs_c2, bs_ra, bs_do;
   // outputs that are not evenly spaced: when set, matrix b writes to c_list[b] / c2_list[b]
   int use_c_list, use_c2_list;
   bf16_t* c_list[kMaxBatch];
@@ -104,6 +105,7 @@ __host__ __device__ inline GemmArgs batch_view(const GemmArgs& g, int b) {
   v.A += b * g.bs_a;
   v.B += b * g.bs_b;
   if (v.E) v.E += b * g.bs_e;
+  if (v.ET) v.ET += b * g.bs_et;
   if (g.use_c_list) v.C = g.c_list[b]; else if (v.C) v.C += b * g.bs_c;
   if (g.use_c2_list) v.C2 = g.c2_list[b]; else if (v.C2) v.C2 += b * g.bs_c2;
   if (v.row_alpha) v.row_alpha += b * g.bs_ra;
