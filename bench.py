@@ -23,12 +23,11 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 DIM = 8192
-# L2-miss traffic of one 8192^2 call (main kernel + the kernel that adds up the split last round),
-# from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
-# 128 MiB device copy (FETCH_SIZE reads half of the copied bytes there, WRITE_SIZE all of them):
-# (505.6e3 + 32.85e3) KiB * 2.0 fetched + (210.1e3 + 3.46e3) KiB written.  The commands and the raw
-# readings are in profiles/syrk_bf16_8192_traffic.md.
-TRAFFIC_BYTES = int((505.6e3 + 32.85e3) * 1024 * 2.0 + (210.1e3 + 3.46e3) * 1024 * 1.0)
+# L2-miss traffic of one 8192^2 call (a single kernel), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a 128 MiB device copy (FETCH_SIZE reads
+# half of the copied bytes there, WRITE_SIZE all of them): 532.7e3 KiB * 2.0 fetched + 148.0e3 KiB
+# written.  The commands and the raw readings are in profiles/syrk_bf16_8192_traffic.md.
+TRAFFIC_BYTES = int(532.7e3 * 1024 * 2.0 + 148.0e3 * 1024 * 1.0)
 
 
 def _time_gpu(fn, steps, warmup, torch):
@@ -258,7 +257,7 @@ def main():
         "effective_tflops": 2.0 * DIM * DIM * DIM / ms / 1e9,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES,
-                     "flop_per_launch": useful, "kernel": "gemm_nt_rounds_kernel (+ gemm_nt_reduce_kernel)"},
+                     "flop_per_launch": useful, "kernel": "gemm_nt_rounds_kernel"},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = _cpu_baseline(X, torch, ns=not args.no_extras, full=args.cpu_full)

@@ -122,8 +122,8 @@ FM_API int fm_syrk_f32(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int
                 int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
- * P = b*A + c*(A*A) for a SYMMETRIC M x M bf16 matrix A (row stride lda).  Same triangular
- * schedule and dual store as fm_syrk_bf16; the polynomial is evaluated on the fp32 accumulator
+ * P = b*A + c*(A*A) for a SYMMETRIC M x M bf16 matrix A (row stride lda; the kernels read A[i][j]
+ * and A[j][i] interchangeably).  Same triangular schedule and dual store as fm_syrk_bf16; the polynomial is evaluated on the fp32 accumulator
  * and rounded to bf16 once.  P must not overlap A.
  * If diag_out is not NULL it receives the M diagonal values of the polynomial in fp32 and the
  * diagonal of P is written as zero: the diagonal carries most of P's magnitude near convergence
@@ -140,8 +140,10 @@ FM_API int fm_syrk_poly_bf16(const void* A, int64_t lda, void* P, int64_t ldp, i
  * Xout = a*X + P*X for P (M x M, row stride ldp) and X (M x K, row stride ldx).  The
  * contraction runs over the rows of X, so the kernel reads X through its transpose
  * XT (K x M, row stride ldxt), which the caller supplies (fm_scale_cast_bf16 and this function
- * both produce it).  Either output may be NULL, not both: Xout is M x K (row stride ldo), XoutT
- * is its transpose K x M (row stride ldot), written from the same registers.
+ * both produce it).  X and XT must hold the same values: on the 256x256 schedule the term a*X is
+ * read through XT as well, on the other schedules through X.  Either output may be NULL, not both:
+ * Xout is M x K (row stride ldo), XoutT is its transpose K x M (row stride ldot), written from the
+ * same registers.
  * If row_alpha is not NULL (M floats), row i uses a + row_alpha[i] in place of a, i.e. the
  * kernel computes a*X + (P + diag(row_alpha))*X with the diagonal term in fp32.
  * No output may overlap an input.
