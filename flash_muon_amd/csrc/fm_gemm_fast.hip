@@ -70,17 +70,22 @@ __device__ __forceinline__ bf16x8_t read_b(const unsigned char* smem, const Frag
   return *reinterpret_cast<const bf16x8_t*>(smem + fa.b[j][ks] + BSLOT * OPER_BYTES);
 }
 
-// one global -> LDS copy with the destination given as an offset from the wave's copy base
+// one global -> LDS copy with the destination given as an offset from the wave's copy base.
+// (s_add_i32 writes SCC: without the clobber the compiler keeps the carry of a 64-bit pointer
+// addition alive across the statement, and a panel that crosses a 4 GiB boundary is then read
+// 4 GiB too low.)
 __device__ __forceinline__ void dma16o(uint32_t voff, const void* sbase, uint32_t lds_base, int off) {
   asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory");
+               :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory", "scc");
 }
 
 // 16 MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The 8 fragment reads of the next
 // substep ride on the first 8, and copies Q0 .. Q1-1 of operand A of the stage two ahead (into the
 // A slot that the previous stage has left) go out between the others, so that the memory pipeline
 // sees an even stream of requests and each of these copies has almost two stages to land.
-template <bool F16, int ASLOT, int BSLOT, int KS, int Q0, int Q1>
+// FIRST: the first substep of a tile, which starts its accumulators from zero instead of having
+// 256 registers cleared beforehand.
+template <bool F16, int ASLOT, int BSLOT, int KS, int Q0, int Q1, bool FIRST = false>
 __device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
                                       const unsigned char* smem, const FragAddr& fa,
                                       const uint32_t (&voA)[8], const bf16_t* gA, uint32_t ldsw) {
@@ -91,7 +96,12 @@ __device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Fr
     else if (q < 8) nxt.b[q - 4] = read_b<BSLOT>(smem, fa, q - 4, KS + 1);
     if (q >= 9 && ((q - 9) & 1) == 0 && Q0 + (q - 9) / 2 < Q1)
       dma16o(voA[Q0 + (q - 9) / 2], gA, ldsw, a_slot_off(AFREE) + (Q0 + (q - 9) / 2) * 4096);
-    FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
+    if constexpr (FIRST) {
+      const f32x16_t zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+      acc[q >> 2][q & 3] = mfma_32x32x16<F16>(cur.a[q >> 2], cur.b[q & 3], zero);
+    } else {
+      FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
+    }
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -120,11 +130,11 @@ __device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cu
 
 // one k stage: the stage in (ASLOT, BSLOT) is multiplied, operand A of the stage two ahead is
 // copied during the first three substeps and operand B of it during the last
-template <bool F16, int ASLOT, int BSLOT>
+template <bool F16, int ASLOT, int BSLOT, bool FIRST = false>
 __device__ __forceinline__ void stage(f32x16_t (&acc)[4][4], Frag& f0, Frag& f1, const unsigned char* smem,
                                       const FragAddr& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
                                       const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
-  phase<F16, ASLOT, BSLOT, 0, 0, 3>(acc, f0, f1, smem, fa, voA, nA, ldsw);
+  phase<F16, ASLOT, BSLOT, 0, 0, 3, FIRST>(acc, f0, f1, smem, fa, voA, nA, ldsw);
   phase<F16, ASLOT, BSLOT, 1, 3, 6>(acc, f1, f0, smem, fa, voA, nA, ldsw);
   phase<F16, ASLOT, BSLOT, 2, 6, 8>(acc, f0, f1, smem, fa, voA, nA, ldsw);
   tail_phase<F16, ASLOT, BSLOT>(acc, f1, f0, smem, fa, voB, nB, ldsw);
@@ -590,10 +600,19 @@ struct FastArgs {
 };
 
 // k stages [kb, ke) of base part `part` of `parts`, or of its sub-part `sub` of `subs`
+// (32-bit arithmetic: nk < 2^15 stages and at most 64 parts; the uncut case costs nothing)
 __device__ __forceinline__ void item_range(int nk, int part, int parts, int sub, int subs, int& kb, int& ke) {
-  const int b0 = (int)((long long)nk * part / parts), b1 = (int)((long long)nk * (part + 1) / parts);
-  kb = b0 + (int)((long long)(b1 - b0) * sub / subs);
-  ke = b0 + (int)((long long)(b1 - b0) * (sub + 1) / subs);
+  unsigned b0 = 0, b1 = (unsigned)nk;
+  if (parts > 1) {
+    b0 = (unsigned)nk * (unsigned)part / (unsigned)parts;
+    b1 = (unsigned)nk * (unsigned)(part + 1) / (unsigned)parts;
+  }
+  kb = (int)b0;
+  ke = (int)b1;
+  if (subs > 1) {
+    kb = (int)(b0 + (b1 - b0) * (unsigned)sub / (unsigned)subs);
+    ke = (int)(b0 + (b1 - b0) * (unsigned)(sub + 1) / (unsigned)subs);
+  }
 }
 
 // Position in the schedule -> tile coordinates.  Tiles are visited in 8x8 blocks (row-major over
@@ -602,9 +621,12 @@ __device__ __forceinline__ void item_range(int nk, int part, int parts, int sub,
 // about 8 + 8 operand panels instead of one panel per tile, and its L2 serves most of the copies.
 __device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& b, int& ti, int& tj) {
   constexpr int SB = 8;
-  const int per_matrix = g.num_tiles / g.batch;
-  b = pos / per_matrix;
-  pos -= b * per_matrix;
+  b = 0;
+  if (g.batch > 1) {
+    const int per_matrix = g.num_tiles / g.batch;
+    b = pos / per_matrix;
+    pos -= b * per_matrix;
+  }
   const int nbm = (g.tiles_m + SB - 1) / SB, nbn = (g.tiles_n + SB - 1) / SB;
   for (int I = 0; I < nbm; ++I) {
     const int rows = (g.tiles_m - I * SB) < SB ? (g.tiles_m - I * SB) : SB;
@@ -806,7 +828,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     if (round < p.rounds) {
       item = round * p.grid + w;
       slot_id = item;
-      item_range(p.nk, item % p.ksplit, p.ksplit, 0, 1, kb, ke);
+      item_range(p.nk, p.ksplit > 1 ? item % p.ksplit : 0, p.ksplit, 0, 1, kb, ke);
     } else if (p.sub64) {
       if (w >= p.rem * 16) break;
       int sbi, sti, stj;
@@ -819,9 +841,9 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       const int j = w / p.split, sub = w - j * p.split;
       item = p.rounds * p.grid + j;
       slot_id = p.tail_slot0 + w;
-      item_range(p.nk, item % p.ksplit, p.ksplit, sub, p.split, kb, ke);
+      item_range(p.nk, p.ksplit > 1 ? item % p.ksplit : 0, p.ksplit, sub, p.split, kb, ke);
     }
-    const int pos = item / p.ksplit;
+    const int pos = p.ksplit > 1 ? item / p.ksplit : item;
     const int n = ke - kb;
     int bi, ti, tj;
     tile_at(p.g, pos, bi, ti, tj);
@@ -841,13 +863,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
     const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
 
-    f32x16_t acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    f32x16_t acc[4][4];   // started from zero by the first substep of the first stage
 
     // ---- main loop over k stages kb .. ke-1 ----------------------------------------------------
     {
@@ -868,34 +884,37 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       __syncthreads();
 #pragma unroll
       for (int q = 0; q < 4; ++q) { f0.a[q] = read_a<0>(smem, fa, q, 0); f0.b[q] = read_b<0>(smem, fa, q, 0); }
-      // the slots come round every 6 stages
-#define FM_STAGE(AS, BS, S)                                                                      \
+      // the slots come round every 6 stages; the first stage stands apart
+#define FM_STAGE_T(AS, BS, S, FIRST)                                                             \
       {                                                                                          \
         const int kn = (S) + 2 < last ? (S) + 2 : last;                                          \
-        stage<F16, AS, BS>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
+        stage<F16, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
       }
-      int s = 0;
+#define FM_STAGE(AS, BS, S) FM_STAGE_T(AS, BS, S, false)
+      FM_STAGE_T(0, 0, 0, true)
+      int s = 1;
       for (; s + 6 <= n; s += 6) {
-        FM_STAGE(0, 0, s)
-        FM_STAGE(1, 1, s + 1)
-        FM_STAGE(2, 0, s + 2)
-        FM_STAGE(0, 1, s + 3)
-        FM_STAGE(1, 0, s + 4)
-        FM_STAGE(2, 1, s + 5)
+        FM_STAGE(1, 1, s)
+        FM_STAGE(2, 0, s + 1)
+        FM_STAGE(0, 1, s + 2)
+        FM_STAGE(1, 0, s + 3)
+        FM_STAGE(2, 1, s + 4)
+        FM_STAGE(0, 0, s + 5)
       }
       if (s < n) {
-        FM_STAGE(0, 0, s)
+        FM_STAGE(1, 1, s)
         if (s + 1 < n) {
-          FM_STAGE(1, 1, s + 1)
+          FM_STAGE(2, 0, s + 1)
           if (s + 2 < n) {
-            FM_STAGE(2, 0, s + 2)
+            FM_STAGE(0, 1, s + 2)
             if (s + 3 < n) {
-              FM_STAGE(0, 1, s + 3)
-              if (s + 4 < n) FM_STAGE(1, 0, s + 4)
+              FM_STAGE(1, 0, s + 3)
+              if (s + 4 < n) FM_STAGE(2, 1, s + 4)
             }
           }
         }
       }
+#undef FM_STAGE_T
 #undef FM_STAGE
       wait_vmcnt<0>();
       __syncthreads();   // no copy in flight and no wave still reading: LDS is free again

@@ -229,3 +229,49 @@ def test_syrk_f16_fast_last_round_in_space(lib, knobs):
     st = lib.fm_syrk_f16(Xd.data_ptr(), 512, Y.data_ptr(), 2048, 1, 2048, 512, None, 0, gpu_util._stream(Xd))
     assert st == 0
     assert torch.equal(Y.cpu(), want)
+
+
+def _across_4gib(big, nbytes, dtype, shape):
+    """A view of `shape` into the byte buffer `big` whose middle lies on a multiple of 4 GiB."""
+    base = big.data_ptr()
+    boundary = (base + 2**32 - 1) // 2**32 * 2**32
+    start = boundary - nbytes // 2
+    assert start >= base and start + nbytes <= base + big.numel() and start % 256 == 0
+    v = big[start - base: start - base + nbytes].view(dtype).view(shape)
+    assert v.data_ptr() < boundary < v.data_ptr() + nbytes
+    return v
+
+
+def test_operands_and_outputs_across_a_4gib_boundary(lib, knobs):
+    """Every operand panel and every output in turn lies across a multiple of 4 GiB, where the low
+    half of its 64-bit addresses wraps: the results are the bits of the same call on tensors that
+    lie elsewhere.  (The copies into LDS take a scalar base and a 32-bit lane offset; a carry lost
+    between the halves of that base reads 4 GiB too low.)"""
+    big = torch.empty(5 * 2**30, dtype=torch.uint8, device=DEV)
+    M, K = 2048, 1024
+    X = _ints((M, K), 77).to(DEV)
+    want = gpu_util.syrk(lib, X)
+    assert torch.equal(want.cpu(), _exact(X.cpu().double() @ X.cpu().double().T))
+    for grid in (-1, 34):                                # whole rounds; sub-tiles in the last round
+        knobs("FLASHMUON_GRID", grid)
+        Xb = _across_4gib(big, M * K * 2, torch.bfloat16, (M, K))
+        Xb.copy_(X)
+        assert torch.equal(gpu_util.syrk(lib, Xb), want)
+        Yb = _across_4gib(big, M * M * 2, torch.bfloat16, (M, M))
+        Yb.fill_(7.0)
+        assert torch.equal(gpu_util.syrk(lib, X, Yb), want)
+    knobs("FLASHMUON_GRID", -1)
+    # the epilogue operand and both outputs of a X + P X
+    M, K = 768, 1536
+    Pm = _ints((M, M), 31, -1, 1).to(DEV)
+    Xs = _ints((M, K), 37).to(DEV)
+    XT = Xs.T.contiguous()
+    Xo, XoT = gpu_util.gemm_axpby(lib, Pm, Xs, 2.0)
+    XTb = _across_4gib(big, M * K * 2, torch.bfloat16, (K, M))
+    XTb.copy_(XT)
+    got = gpu_util.gemm_axpby(lib, Pm, Xs, 2.0, XT=XTb)
+    assert torch.equal(got[0], Xo) and torch.equal(got[1], XoT)
+    Pb = _across_4gib(big, M * M * 2, torch.bfloat16, (M, M))
+    Pb.copy_(Pm)
+    got = gpu_util.gemm_axpby(lib, Pb, Xs, 2.0)
+    assert torch.equal(got[0], Xo) and torch.equal(got[1], XoT)
