@@ -366,18 +366,21 @@ __device__ __forceinline__ void epilogue_quarter(const GemmArgs& g, bool diag, f
 
 // ---- write-out of a whole tile from the accumulators --------------------------------------------
 // An MFMA accumulator register pair of a lane holds two consecutive rows of one column, which is
-// what the transposed output wants: after rounding, the pairs go to C2 straight from the
-// registers (two lanes 32 apart swap halves first, so that every lane stores 8 consecutive rows,
-// 16 bytes).  Only the direct output needs the transposition through LDS, and it stages the rounded
-// 16-bit values: neighbouring lanes (columns c and c+1) exchange halves, so that every lane holds
-// two consecutive columns of one row, and a quarter (32 rows x 128 columns) is staged row-major,
-// 8 KiB instead of 16 KiB of fp32, and read back 16 bytes per lane.  Both copies carry the same bits.
+// what the transposed output wants: after rounding, a lane has 8 bytes of a row of C2 per register
+// quadruple.  They are collected column by column in LDS over two quarters (64 rows = 128 bytes per
+// column) and leave as whole cache lines, 8 lanes per row of C2.  The direct output needs a real
+// transposition, and it stages the same rounded 16-bit values: neighbouring lanes (columns c and
+// c+1) exchange halves, so that every lane holds two consecutive columns of one row, and a quarter
+// (32 rows x 128 columns) is staged row-major, 8 KiB instead of 16 KiB of fp32, and read back 16
+// bytes per lane.  Both copies carry the same bits.
 // The operand E is read transposed (ET) in the accumulators' own layout, 8 consecutive rows of one
 // column per lane and load, so the arithmetic happens in registers before anything is staged.
 constexpr int QT_PITCH = 320;             // bytes per staged row: 128 values + 64 bytes, so that rows r and r+1 use different banks
 constexpr int QT_BYTES = 32 * QT_PITCH;   // one staged quarter of a wave
-constexpr int QS_OFFSET = QT_BYTES + 512; // after it the row additions, then the quarter's accumulators (16 KiB)
-static_assert(QS_OFFSET + 16 * 1024 <= EPI_WAVE_BYTES, "the write-out stages inside the wave's region");
+constexpr int QM_PITCH = 136;             // bytes per staged column of the mirrored copy: 64 rows + 8 bytes (2-way conflicts at most)
+constexpr int QM_OFFSET = QT_BYTES + 512; // after the direct staging and the 128 row additions
+constexpr int QM_BYTES = 128 * QM_PITCH;  // two quarters of the mirrored copy
+static_assert(QM_OFFSET + QM_BYTES <= EPI_WAVE_BYTES, "the write-out stages inside the wave's region");
 
 // 16 bytes per lane at base + voff + soff (bytes) through a buffer descriptor: the per-lane part of
 // an address is one 32-bit register, the rest is scalar
@@ -451,12 +454,15 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
   // rows 32i + 16t + 8lh .. +7 of column 32j + lc are what a lane loads of ET and stores to C2,
   // row 4it + lane/16, columns 8(lane % 16) .. +7 what it stores to C.
   const uint32_t et_lane = (uint32_t)(lc * (int)g.ldet + 8 * lh) * 2u;
-  const uint32_t c2_lane = (uint32_t)(lc * (int)g.c2_rs + 8 * lh) * 2u;
+  // rows 64h + 8(lane % 8) .. +7 of column 8it + lane/8: the mirrored copy, a cache line per 8 lanes
+  const uint32_t c2_lane = (uint32_t)((lane >> 3) * (int)g.c2_rs + (lane & 7) * 8) * 2u;
+  unsigned char* const mw = T + QM_OFFSET + lc * QM_PITCH + 8 * lh;
+  const unsigned char* const mr = T + QM_OFFSET + (lane >> 3) * QM_PITCH + (lane & 7) * 16;
   const uint32_t c_lane = (uint32_t)((lane >> 4) * (int)g.c_rs + (lane & 15) * 8) * 2u;
   const __amdgpu_buffer_rsrc_t et_buf = block_rsrc(g.ET + (int64_t)col0 * g.ldet + row0);
   const __amdgpu_buffer_rsrc_t c2_buf = block_rsrc(g.C2 + (int64_t)col0 * g.c2_rs + row0);
   const __amdgpu_buffer_rsrc_t c_buf = block_rsrc(g.C + (int64_t)row0 * g.c_rs + col0);
-  const int et_col = 64 * (int)g.ldet, c2_col = 64 * (int)g.c2_rs, c_row = 8 * (int)g.c_rs;   // bytes: 32 columns, 32 columns, 4 rows
+  const int et_col = 64 * (int)g.ldet, c2_col = 16 * (int)g.c2_rs, c_row = 8 * (int)g.c_rs;   // bytes: 32 columns, 8 columns, 4 rows
 #define FM_ET(i, j, t) buf_load16(et_buf, et_lane, (j) * et_col + 64 * (i) + 32 * (t))
 
   uint4 ev[4][2];
@@ -540,14 +546,10 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
             *reinterpret_cast<uint32_t*>(tw + (8 * qq + 2 * h) * QT_PITCH + 64 * j) = __builtin_amdgcn_perm(nbr, own, sel);
           }
       }
-      if (mirror) {
+      if (mirror) {   // rows 32(i % 2) + 8qq + 4lh .. +3 of column 32j + lc, for the pass after every second quarter
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          uint4 o = {P[2 * t][0], P[2 * t][1], P[2 * t + 1][0], P[2 * t + 1][1]};
-          swap32(o.x, o.z);   // now rows 16t + 8lh .. +7, in the order x y z w
-          swap32(o.y, o.w);
-          buf_store16(c2_buf, c2_lane, j * c2_col + 64 * i + 32 * t, o);
-        }
+        for (int qq = 0; qq < 4; ++qq)
+          *reinterpret_cast<uint2*>(mw + 32 * j * QM_PITCH + 64 * (i & 1) + 16 * qq) = uint2{P[qq][0], P[qq][1]};
       }
       };
       if (i == j && dout) tile(std::true_type{});
@@ -570,6 +572,22 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
         for (int it = 0; it < 4; ++it) d[it] = *reinterpret_cast<const uint4*>(tr + 4 * (4 * half + it) * QT_PITCH);
 #pragma unroll
         for (int it = 0; it < 4; ++it) buf_store16(c_buf, c_lane, (8 * i + 4 * half + it) * c_row, d[it]);
+      }
+    }
+    if (mirror && (i & 1)) {   // two quarters of the mirrored copy: 128 columns x 128 bytes
+#pragma unroll
+      for (int grp = 0; grp < 4; ++grp) {
+        uint2 d[4][2];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const unsigned char* src = mr + 8 * (4 * grp + it) * QM_PITCH;
+          d[it][0] = *reinterpret_cast<const uint2*>(src);
+          d[it][1] = *reinterpret_cast<const uint2*>(src + 8);
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+          buf_store16(c2_buf, c2_lane, (4 * grp + it) * c2_col + 128 * (i >> 1),
+                      uint4{d[it][0].x, d[it][0].y, d[it][1].x, d[it][1].y});
       }
     }
   }
