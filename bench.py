@@ -25,9 +25,9 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 DIM = 8192
 # L2-miss traffic of one 8192^2 call (a single kernel), from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the same counter reads for a 128 MiB device copy (FETCH_SIZE reads
-# half of the copied bytes there, WRITE_SIZE all of them): 532.7e3 KiB * 2.0 fetched + 148.0e3 KiB
+# half of the copied bytes there, WRITE_SIZE all of them): 508.3e3 KiB * 2.0 fetched + 131.1e3 KiB
 # written.  The commands and the raw readings are in profiles/syrk_bf16_8192_traffic.md.
-TRAFFIC_BYTES = int(532.7e3 * 1024 * 2.0 + 148.0e3 * 1024 * 1.0)
+TRAFFIC_BYTES = int(508.3e3 * 1024 * 2.0 + 131.1e3 * 1024 * 1.0)
 
 
 def _time_gpu(fn, steps, warmup, torch):
