@@ -160,6 +160,13 @@ def _extras(Xd, steps, warmup, torch):
         ex["xxt_%d_useful_tflops" % dim] = synthetic.syrk_useful_flop(dim, dim) / ours / 1e9
         ex["torch_xxt_%d_ms" % dim] = ref
         ex["xxt_%d_speedup_vs_torch" % dim] = ref / ours
+        # W + K calls of these sizes last a few milliseconds and fall into the power-management
+        # transient after idle; the same pair once more over 100 + 200 calls each
+        ours_s = _time_gpu(lambda: matmul_transpose(Xs), 200, 100, torch)
+        ref_s = _time_gpu(lambda: torch.matmul(Xs, Xs.T), 200, 100, torch)
+        ex["xxt_%d_steady_ms" % dim] = ours_s
+        ex["torch_xxt_%d_steady_ms" % dim] = ref_s
+        ex["xxt_%d_steady_speedup_vs_torch" % dim] = ref_s / ours_s
         del Xs
     # fast_newtonschulz(5) on the gradient-like inputs of the rectangular and the square case
     # (noise of std 1e-3 plus a rank-r spike, Frobenius-normalised; generated on the CPU from the
