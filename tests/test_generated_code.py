@@ -1,0 +1,99 @@
+"""Checks on the machine code hipcc generates for the hand-scheduled GEMM kernels (no GPU needed):
+what the compiler may not know about the inline assembly, it must be told.
+
+The copies into LDS are inline assembly because the compiler would otherwise wait for all of them in
+front of every LDS read.  The price is that the compiler trusts the statement's clobber list: an
+`s_add_i32` inside it writes SCC, and when the list did not say so one build kept the carry of a
+64-bit pointer addition alive across a copy (`s_add_u32`, copy, `s_addc_u32`), which reads an operand
+panel that crosses a 4 GiB boundary 4 GiB too low.  These tests look for that pattern, and for
+spills, in the code as built."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from flash_muon_amd import build
+
+SRC = os.path.join(build.CSRC, "fm_gemm_fast.hip")
+
+# scalar ALU operations that write SCC (all but moves, multiplies and a few others do)
+_SCC_WRITERS = re.compile(
+    r"^(s_add_[iu]32|s_sub_[iu]32|s_addc_u32|s_subb_u32|s_cmp\w*|s_bitcmp\w*|s_and\w*|s_or\w*|s_xor\w*|s_nand\w*|"
+    r"s_nor\w*|s_xnor\w*|s_not\w*|s_lshl\w*|s_lshr\w*|s_ashr\w*|s_min_[iu]32|s_max_[iu]32|s_abs\w*|s_bfe\w*|"
+    r"s_absdiff\w*|s_wqm\w*|s_quadmask\w*|s_bcnt\w*)\b")
+_SCC_READERS = re.compile(r"^(s_addc_u32|s_subb_u32|s_cselect_b(32|64)|s_cbranch_scc[01]|s_cmov\w*)\b")
+
+
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    if shutil.which(build.HIPCC) is None and not os.path.exists(build.HIPCC):
+        pytest.skip("no hipcc here")
+    out = tmp_path_factory.mktemp("asm") / "fm_gemm_fast.s"
+    cmd = [build.HIPCC, *[f for f in build.FLAGS if f != "-fPIC"], "-S", "--cuda-device-only", SRC, "-o", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return out.read_text().split("\n")
+
+
+def _is_code(t):
+    return bool(t) and not t.startswith(";") and not t.startswith(".") and not t.endswith(":")
+
+
+def test_no_scc_value_lives_across_an_assembly_statement_that_writes_scc(assembly):
+    kernel, in_asm, scc_set_at, clobbered_at, found = None, False, None, None, []
+    for i, line in enumerate(assembly):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            kernel, scc_set_at, clobbered_at = m.group(1), None, None
+        t = line.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if t.endswith(":") and not t.startswith(";"):      # a new basic block: what is live is not followed further
+            scc_set_at, clobbered_at = None, None
+            continue
+        if not _is_code(t):
+            continue
+        if in_asm:
+            if _SCC_WRITERS.match(t) and scc_set_at is not None:
+                clobbered_at = i + 1
+            continue
+        if _SCC_READERS.match(t) and scc_set_at is not None and clobbered_at is not None:
+            found.append("%s: SCC set in line %d, overwritten inside an asm statement in line %d, read in line %d (%s)"
+                         % (kernel, scc_set_at, clobbered_at, i + 1, t))
+        if _SCC_WRITERS.match(t):
+            scc_set_at, clobbered_at = i + 1, None
+    assert not found, "\n".join(found)
+
+
+def test_every_assembly_statement_that_writes_scc_says_so():
+    text = open(SRC).read()
+    bad = []
+    for m in re.finditer(r"asm volatile\((.*?)\);", text, re.S):
+        body = m.group(1)
+        instrs = re.findall(r"\b(s_[a-z0-9_]+)\b", body.split("::")[0] if "::" in body else body)
+        if any(_SCC_WRITERS.match(x) for x in instrs) and '"scc"' not in body:
+            bad.append(body.strip().split("\n")[0][:100])
+    assert not bad, bad
+
+
+def test_gemm_kernels_do_not_spill(assembly):
+    """One wave per SIMD owns all 512 registers of a lane; a spill means scratch traffic inside the
+    MFMA loop or the write-out."""
+    sizes = {}
+    kernel = None
+    for line in assembly:
+        m = re.match(r"\s*\.amdhsa_kernel\s+(\S+)", line)
+        if m:
+            kernel = m.group(1)
+        m = re.match(r"\s*\.amdhsa_private_segment_fixed_size\s+(\d+)", line)
+        if m and kernel:
+            sizes[kernel] = int(m.group(1))
+    gemm = {k: v for k, v in sizes.items() if "gemm_nt" in k}
+    assert len(gemm) >= 6, sorted(sizes)           # rounds x 4 instances, reduce x 2, mid x 2
+    assert all(v == 0 for v in gemm.values()), {k: v for k, v in gemm.items() if v}
