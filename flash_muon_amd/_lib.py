@@ -15,7 +15,7 @@ FM_OK = 0
 FM_ERR_STRIDE = 3
 FM_ERR_ALIAS = 5
 # fm_knob values
-FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID, FM_KNOB_NO_SUB64 = 0, 1, 2, 3, 4
+FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID, FM_KNOB_NO_SUB64, FM_KNOB_HALF = 0, 1, 2, 3, 4, 5
 FM_BF16, FM_F16, FM_F32 = 0, 1, 2
 
 _DTYPE_CODE = {torch.bfloat16: FM_BF16, torch.float16: FM_F16, torch.float32: FM_F32}

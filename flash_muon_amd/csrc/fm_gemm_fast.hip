@@ -41,7 +41,9 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
 
 #define FM_MFMA(i, j, FA, FB) acc[i][j] = mfma_32x32x16<F16>(FA[i], FB[j], acc[i][j])
 
-struct Frag { bf16x8_t a[4], b[4]; };
+// NI: rows of 32x32 MFMA tiles per wave.  4: a wave computes 128x128 of a 256x256 tile; 2: 64x128
+// of a 128x256 half tile (operand A is then half as tall and uses half of each of its slots).
+template <int NI> struct Frag { bf16x8_t a[NI], b[4]; };
 
 // LDS during the main loop: three stages of operand A and two of operand B, 32 KiB each, in the
 // order A0 A1 B0 B1 A2.  Stage s of A sits in A slot s % 3, stage s of B in B slot s % 2.  A
@@ -49,24 +51,23 @@ struct Frag { bf16x8_t a[4], b[4]; };
 // the fragment addresses are kept for the windows at 0 (A0, A1), 64 KiB (B0, B1) and 128 KiB (A2)
 // and no address arithmetic is left in the loop (every VALU instruction between two MFMAs delays
 // the second one by its own issue time).
-constexpr int A_SLOTS = 3, B_SLOTS = 2;
 __host__ __device__ constexpr int a_slot_off(int slot) { return slot == 2 ? 4 * OPER_BYTES : slot * OPER_BYTES; }
 __host__ __device__ constexpr int b_slot_off(int slot) { return (2 + slot) * OPER_BYTES; }
 
 // per-lane LDS byte addresses of the fragments: [window][fragment][k16 substep]
-struct FragAddr {
-  uint32_t a_lo[4][4];   // A rows, slots 0 and 1 (offset 0 / OPER_BYTES)
-  uint32_t a_hi[4][4];   // A rows, slot 2
+template <int NI> struct FragAddr {
+  uint32_t a_lo[NI][4];  // A rows, slots 0 and 1 (offset 0 / OPER_BYTES)
+  uint32_t a_hi[NI][4];  // A rows, slot 2
   uint32_t b[4][4];      // B rows, B slots 0 and 1 (offset 0 / OPER_BYTES from the window at 64 KiB)
 };
 
-template <int ASLOT>
-__device__ __forceinline__ bf16x8_t read_a(const unsigned char* smem, const FragAddr& fa, int i, int ks) {
+template <int ASLOT, int NI>
+__device__ __forceinline__ bf16x8_t read_a(const unsigned char* smem, const FragAddr<NI>& fa, int i, int ks) {
   if constexpr (ASLOT == 2) return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_hi[i][ks]);
   else return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_lo[i][ks] + ASLOT * OPER_BYTES);
 }
-template <int BSLOT>
-__device__ __forceinline__ bf16x8_t read_b(const unsigned char* smem, const FragAddr& fa, int j, int ks) {
+template <int BSLOT, int NI>
+__device__ __forceinline__ bf16x8_t read_b(const unsigned char* smem, const FragAddr<NI>& fa, int j, int ks) {
   return *reinterpret_cast<const bf16x8_t*>(smem + fa.b[j][ks] + BSLOT * OPER_BYTES);
 }
 
@@ -79,23 +80,25 @@ __device__ __forceinline__ void dma16o(uint32_t voff, const void* sbase, uint32_
                :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory", "scc");
 }
 
-// 16 MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The 8 fragment reads of the next
-// substep ride on the first 8, and copies Q0 .. Q1-1 of operand A of the stage two ahead (into the
-// A slot that the previous stage has left) go out between the others, so that the memory pipeline
-// sees an even stream of requests and each of these copies has almost two stages to land.
+// The 4 NI MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The NI + 4 fragment reads of
+// the next substep ride on the first ones, and copies Q0 .. Q1-1 of operand A of the stage two
+// ahead (into the A slot that the previous stage has left) go out between the others, so that the
+// memory pipeline sees an even stream of requests and each of these copies has almost two stages
+// to land.
 // FIRST: the first substep of a tile, which starts its accumulators from zero instead of having
-// 256 registers cleared beforehand.
-template <bool F16, int ASLOT, int BSLOT, int KS, int Q0, int Q1, bool FIRST = false>
-__device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
-                                      const unsigned char* smem, const FragAddr& fa,
-                                      const uint32_t (&voA)[8], const bf16_t* gA, uint32_t ldsw) {
+// the registers cleared beforehand.
+template <bool F16, int NI, int ASLOT, int BSLOT, int KS, int Q0, int Q1, bool FIRST = false, int NR>
+__device__ __forceinline__ void phase(f32x16_t (&acc)[NR][4], const Frag<NI>& cur, Frag<NI>& nxt,
+                                      const unsigned char* smem, const FragAddr<NI>& fa,
+                                      const uint32_t (&voA)[2 * NI], const bf16_t* gA, uint32_t ldsw) {
   constexpr int AFREE = (ASLOT + 2) % 3;
+  constexpr int DQ0 = NI == 4 ? 9 : 6, DSTEP = NI == 4 ? 2 : 1;   // where the copies go: after the reads
 #pragma unroll
-  for (int q = 0; q < 16; ++q) {
-    if (q < 4) nxt.a[q] = read_a<ASLOT>(smem, fa, q, KS + 1);
-    else if (q < 8) nxt.b[q - 4] = read_b<BSLOT>(smem, fa, q - 4, KS + 1);
-    if (q >= 9 && ((q - 9) & 1) == 0 && Q0 + (q - 9) / 2 < Q1)
-      dma16o(voA[Q0 + (q - 9) / 2], gA, ldsw, a_slot_off(AFREE) + (Q0 + (q - 9) / 2) * 4096);
+  for (int q = 0; q < 4 * NI; ++q) {
+    if (q < NI) nxt.a[q] = read_a<ASLOT>(smem, fa, q, KS + 1);
+    else if (q < NI + 4) nxt.b[q - NI] = read_b<BSLOT>(smem, fa, q - NI, KS + 1);
+    if (q >= DQ0 && (q - DQ0) % DSTEP == 0 && Q0 + (q - DQ0) / DSTEP < Q1)
+      dma16o(voA[Q0 + (q - DQ0) / DSTEP], gA, ldsw, a_slot_off(AFREE) + (Q0 + (q - DQ0) / DSTEP) * 4096);
     if constexpr (FIRST) {
       const f32x16_t zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
       acc[q >> 2][q & 3] = mfma_32x32x16<F16>(cur.a[q >> 2], cur.b[q & 3], zero);
@@ -107,22 +110,23 @@ __device__ __forceinline__ void phase(f32x16_t (&acc)[4][4], const Frag& cur, Fr
 }
 
 // Last substep of a stage.  Before it every wave waits for its copies of the next stage (all but
-// the 8 newest, which belong to the stage after) and, at the barrier, for everybody else's; then
-// the 16 MFMAs run interleaved with the 8 copies of operand B two stages ahead, into the B slot
+// the 2 NI newest, which belong to the stage after) and, at the barrier, for everybody else's; then
+// the MFMAs run interleaved with the 8 copies of operand B two stages ahead, into the B slot
 // this stage has just left, and with the first fragment reads of the next stage.
-template <bool F16, int ASLOT, int BSLOT>
-__device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cur, Frag& nxt,
-                                           const unsigned char* smem, const FragAddr& fa,
+template <bool F16, int NI, int ASLOT, int BSLOT, int NR>
+__device__ __forceinline__ void tail_phase(f32x16_t (&acc)[NR][4], const Frag<NI>& cur, Frag<NI>& nxt,
+                                           const unsigned char* smem, const FragAddr<NI>& fa,
                                            const uint32_t (&voB)[8], const bf16_t* gB, uint32_t ldsw) {
   constexpr int ANEXT = (ASLOT + 1) % 3, BNEXT = BSLOT ^ 1;
+  constexpr int BSTEP = NI / 2;   // MFMAs per copy of operand B
   // (the fragment reads of this stage were issued a substep ago; lgkmcnt(0) makes it formal that
   // nobody still reads the slots that are about to be refilled)
-  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(2 * NI) : "memory");
 #pragma unroll
-  for (int q = 0; q < 16; ++q) {
-    if ((q & 1) == 0) dma16o(voB[q >> 1], gB, ldsw, b_slot_off(BSLOT) + (q >> 1) * 4096);
-    if (q < 4) nxt.a[q] = read_a<ANEXT>(smem, fa, q, 0);
-    else if (q < 8) nxt.b[q - 4] = read_b<BNEXT>(smem, fa, q - 4, 0);
+  for (int q = 0; q < 4 * NI; ++q) {
+    if (q % BSTEP == 0) dma16o(voB[q / BSTEP], gB, ldsw, b_slot_off(BSLOT) + (q / BSTEP) * 4096);
+    if (q < NI) nxt.a[q] = read_a<ANEXT>(smem, fa, q, 0);
+    else if (q < NI + 4) nxt.b[q - NI] = read_b<BNEXT>(smem, fa, q - NI, 0);
     FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -130,14 +134,77 @@ __device__ __forceinline__ void tail_phase(f32x16_t (&acc)[4][4], const Frag& cu
 
 // one k stage: the stage in (ASLOT, BSLOT) is multiplied, operand A of the stage two ahead is
 // copied during the first three substeps and operand B of it during the last
-template <bool F16, int ASLOT, int BSLOT, bool FIRST = false>
-__device__ __forceinline__ void stage(f32x16_t (&acc)[4][4], Frag& f0, Frag& f1, const unsigned char* smem,
-                                      const FragAddr& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+template <bool F16, int NI, int ASLOT, int BSLOT, bool FIRST = false, int NR>
+__device__ __forceinline__ void stage(f32x16_t (&acc)[NR][4], Frag<NI>& f0, Frag<NI>& f1, const unsigned char* smem,
+                                      const FragAddr<NI>& fa, const uint32_t (&voA)[2 * NI], const uint32_t (&voB)[8],
                                       const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
-  phase<F16, ASLOT, BSLOT, 0, 0, 3, FIRST>(acc, f0, f1, smem, fa, voA, nA, ldsw);
-  phase<F16, ASLOT, BSLOT, 1, 3, 6>(acc, f1, f0, smem, fa, voA, nA, ldsw);
-  phase<F16, ASLOT, BSLOT, 2, 6, 8>(acc, f0, f1, smem, fa, voA, nA, ldsw);
-  tail_phase<F16, ASLOT, BSLOT>(acc, f1, f0, smem, fa, voB, nB, ldsw);
+  constexpr int Q1 = NI == 4 ? 3 : 2, Q2 = NI == 4 ? 6 : 3;   // the 2 NI copies of operand A over three substeps
+  phase<F16, NI, ASLOT, BSLOT, 0, 0, Q1, FIRST>(acc, f0, f1, smem, fa, voA, nA, ldsw);
+  phase<F16, NI, ASLOT, BSLOT, 1, Q1, Q2>(acc, f1, f0, smem, fa, voA, nA, ldsw);
+  phase<F16, NI, ASLOT, BSLOT, 2, Q2, 2 * NI>(acc, f0, f1, smem, fa, voA, nA, ldsw);
+  tail_phase<F16, NI, ASLOT, BSLOT>(acc, f1, f0, smem, fa, voB, nB, ldsw);
+}
+
+// ---- a diagonal tile of a symmetric product as one item of the half-tile schedule ---------------
+// Of the 8 x 8 MFMA tiles of a diagonal 256x256 tile only those on or below the diagonal are
+// distinct: 36, against the 32 of a half tile.  They are shared out 10, 10, 8, 8: waves 0 and 1
+// take the lower triangles of the two 128x128 squares on the diagonal (4 fragments, 10 MFMAs per
+// substep), waves 2 and 3 a 64x128 half each of the square above the diagonal, in the shape of any
+// other wave of the half-tile kernel.  Both operands are the one 256-row panel, which goes round
+// the three A slots (8 copies per wave and stage, issued two stages ahead); the B slots are idle.
+struct DFrag { bf16x8_t f[6]; };   // triangle waves: rows 32q of their square; the others: 2 row and 4 column fragments
+struct DFragAddr { uint32_t lo[6][4], hi[6][4]; };   // A slots 0 and 1 / A slot 2
+
+template <int ASLOT>
+__device__ __forceinline__ bf16x8_t read_d(const unsigned char* smem, const DFragAddr& fa, int q, int ks) {
+  if constexpr (ASLOT == 2) return *reinterpret_cast<const bf16x8_t*>(smem + fa.hi[q][ks]);
+  else return *reinterpret_cast<const bf16x8_t*>(smem + fa.lo[q][ks] + ASLOT * OPER_BYTES);
+}
+
+// where a triangle wave keeps MFMA tile (i, j), j <= i, among its 3 x 4 accumulator tuples
+__host__ __device__ constexpr int tri_r(int i, int j) { return i < 3 ? i : (j < 3 ? 0 : 1); }
+__host__ __device__ constexpr int tri_c(int i, int j) { return i < 3 ? j : (j < 3 ? j + 1 : 2); }
+// row and column fragment of MFMA q of a triangle wave, in the order (0,0) (1,0) (1,1) (2,0) ...
+__host__ __device__ constexpr int tri_i(int q) { return q < 1 ? 0 : q < 3 ? 1 : q < 6 ? 2 : 3; }
+__host__ __device__ constexpr int tri_j(int q) { return q - tri_i(q) * (tri_i(q) + 1) / 2; }
+
+// the MFMAs of one substep: 10 (TRI) or 8, with READS fragment reads of `ks_next` of slot RSLOT
+// riding on the first ones and copies Q0 .. Q1-1 of the panel two stages ahead on the later ones
+template <bool F16, bool TRI, int RSLOT, int Q0, int Q1, int CSLOT, bool FIRST>
+__device__ __forceinline__ void dsubstep(f32x16_t (&acc)[3][4], const DFrag& cur, DFrag& nxt, const unsigned char* smem,
+                                         const DFragAddr& fa, int ks_next, const uint32_t (&vo)[8], const bf16_t* gP,
+                                         uint32_t ldsw) {
+  constexpr int NM = TRI ? 10 : 8, NRD = TRI ? 4 : 6;
+  constexpr int C0 = 5, CSTEP = TRI ? 2 : 1;   // copies after MFMA 5, 7, 9 or 5, 6, 7
+#pragma unroll
+  for (int q = 0; q < NM; ++q) {
+    if (q < NRD) nxt.f[q] = read_d<RSLOT>(smem, fa, q, ks_next);
+    if (q >= C0 && (q - C0) % CSTEP == 0 && Q0 + (q - C0) / CSTEP < Q1)
+      dma16o(vo[Q0 + (q - C0) / CSTEP], gP, ldsw, a_slot_off(CSLOT) + (Q0 + (q - C0) / CSTEP) * 4096);
+    const f32x16_t zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if constexpr (TRI) {
+      f32x16_t& c = acc[tri_r(tri_i(q), tri_j(q))][tri_c(tri_i(q), tri_j(q))];
+      c = mfma_32x32x16<F16>(cur.f[tri_i(q)], cur.f[tri_j(q)], FIRST ? zero : c);
+    } else {
+      f32x16_t& c = acc[q >> 2][q & 3];
+      c = mfma_32x32x16<F16>(cur.f[q >> 2], cur.f[2 + (q & 3)], FIRST ? zero : c);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// one k stage of the panel in A slot ASLOT
+template <bool F16, bool TRI, int ASLOT, bool FIRST>
+__device__ __forceinline__ void dstage(f32x16_t (&acc)[3][4], DFrag& f0, DFrag& f1, const unsigned char* smem,
+                                       const DFragAddr& fa, const uint32_t (&vo)[8], const bf16_t* nP, uint32_t ldsw) {
+  constexpr int AFREE = (ASLOT + 2) % 3, ANEXT = (ASLOT + 1) % 3;
+  dsubstep<F16, TRI, ASLOT, 0, 3, AFREE, FIRST>(acc, f0, f1, smem, fa, 1, vo, nP, ldsw);
+  dsubstep<F16, TRI, ASLOT, 3, 6, AFREE, false>(acc, f1, f0, smem, fa, 2, vo, nP, ldsw);
+  dsubstep<F16, TRI, ASLOT, 6, 8, AFREE, false>(acc, f0, f1, smem, fa, 3, vo, nP, ldsw);
+  // everybody's copies of the next stage have landed (all but the 8 newest, of the stage after),
+  // and nobody reads the slot that the next stage's copies go to
+  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  dsubstep<F16, TRI, ANEXT, 0, 0, AFREE, false>(acc, f1, f0, smem, fa, 0, vo, nP, ldsw);
 }
 
 // ---- the part of a tile after the main loop -----------------------------------------------------
@@ -397,14 +464,6 @@ __device__ __forceinline__ void buf_store16(__amdgpu_buffer_rsrc_t b, uint32_t v
   __builtin_amdgcn_raw_buffer_store_b128(v, b, (int)voff, soff, 0);
 }
 
-// One accumulator element, copied out of the accumulator file at this point of the program: left
-// to the compiler, all 256 are copied where the main loop ends, and do not fit.
-__device__ __forceinline__ float acc_read(float a) {
-  float v;
-  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(a));
-  return v;
-}
-
 __device__ __forceinline__ void swap32(uint32_t& lo_half_keeps, uint32_t& hi_half_keeps) {
   // lanes 0..31 give `hi_half_keeps` to, and take `lo_half_keeps` of, the lane 32 above
   const auto r = __builtin_amdgcn_permlane32_swap(lo_half_keeps, hi_half_keeps, false, false);
@@ -430,10 +489,17 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 // and any beta.  A kernel holds one instance only: of identical element reads in several branches
 // the optimizer makes one read of all 256 accumulators ahead of the branch, and they do not fit
 // into the vector registers.
-template <bool F16, int MODE>
-__device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool diag_block,
-                                              const f32x16_t (&acc)[4][4], unsigned char* T, int row0, int col0,
+// The wave's block is 32 NI rows x 128 columns at (row0, col0).  `diag`: the block has no mirror
+// image to write (it lies in a diagonal tile of a symmetric product, which holds both); `dshift`:
+// MFMA tile (i, i + dshift) of the block lies on the diagonal of the output, or a value no tile has.
+// TRI: the block is a 128x128 square on the diagonal of a symmetric product of which the wave
+// holds the MFMA tiles (i, j), j <= i, at acc[tri_r(i, j)][tri_c(i, j)]: those are written in
+// place, and the ones below the diagonal also as their mirror images above it.
+template <bool F16, int MODE, int NI, bool TRI, int NR>
+__device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int dshift,
+                                              const f32x16_t (&acc)[NR][4], unsigned char* T, int row0, int col0,
                                               int lane) {
+  constexpr int NQ = TRI ? 4 : NI;   // quarters: rows of MFMA tiles
   // what follows is derived from `lane` anew for every tile: kept in registers across the main
   // loop instead, the per-lane offsets of the write-out would crowd out the loop's own
   asm volatile("" : "+v"(lane));
@@ -441,7 +507,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
   const int lc = lane & 31, lh = lane >> 5, par = lane & 1;
   const bool direct = g.C != nullptr;
   const bool mirror = g.C2 != nullptr && !diag;
-  const bool dout = diag && diag_block && g.diag_out != nullptr;
+  const bool dout = (TRI || diag) && g.diag_out != nullptr;
   const float alpha = g.alpha, beta = g.beta;
   const uint32_t sel = par ? 0x03020706u : 0x05040100u;   // odd lanes keep the high halves, even lanes the low ones
   float* const RA = reinterpret_cast<float*>(T + QT_BYTES);
@@ -467,18 +533,20 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
 
   uint4 ev[4][2];
   if constexpr (has_e) {
-    // the block's 128 additions to alpha (zeros when there are none), before any store of this tile
+    // the block's 32 NI additions to alpha (zeros when there are none), before any store of this tile
     float2 ra = {0.0f, 0.0f};
-    if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
-    *reinterpret_cast<float2*>(RA + lane * 2) = ra;
+    if (NQ == 4 || lane < 16 * NQ) {
+      if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+      *reinterpret_cast<float2*>(RA + lane * 2) = ra;
+    }
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < (TRI ? 1 : 4); ++j)
 #pragma unroll
       for (int t = 0; t < 2; ++t) ev[j][t] = FM_ET(0, j, t);
   }
 
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < NQ; ++i) {
     f32x4_t al[4];
     if constexpr (has_e) {
 #pragma unroll
@@ -489,7 +557,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < (TRI ? i + 1 : 4); ++j) {
       // the scheduler works on one MFMA tile at a time: left alone with the whole unrolled
       // write-out, it moves every accumulator to a vector register first and runs out of them
       __builtin_amdgcn_sched_barrier(0);
@@ -499,7 +567,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
       constexpr bool DOUT = decltype(dout_tag)::value;
       float v[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) v[r] = acc[i][j][r];
+      for (int r = 0; r < 16; ++r) v[r] = acc[TRI ? tri_r(i, j) : i][TRI ? tri_c(i, j) : j][r];
       if constexpr (has_e) {
         uint32_t eb[4][2];   // [qq][h]: the operand in the accumulators' layout
 #pragma unroll
@@ -508,7 +576,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
           swap32(a0, b0);
           swap32(a1, b1);
           eb[2 * t][0] = a0; eb[2 * t][1] = a1; eb[2 * t + 1][0] = b0; eb[2 * t + 1][1] = b1;
-          if (i < 3) ev[j][t] = FM_ET(i + 1, j, t);
+          if (i < NQ - 1) ev[j][t] = FM_ET(i + 1, j, t);
         }
         if constexpr (MODE == 2) {
 #pragma unroll
@@ -546,13 +614,13 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
             *reinterpret_cast<uint32_t*>(tw + (8 * qq + 2 * h) * QT_PITCH + 64 * j) = __builtin_amdgcn_perm(nbr, own, sel);
           }
       }
-      if (mirror) {   // rows 32(i % 2) + 8qq + 4lh .. +3 of column 32j + lc, for the pass after every second quarter
+      if (mirror && (!TRI || j < i)) {   // rows 32(i % 2) + 8qq + 4lh .. +3 of column 32j + lc, for the pass after every second quarter
 #pragma unroll
         for (int qq = 0; qq < 4; ++qq)
           *reinterpret_cast<uint2*>(mw + 32 * j * QM_PITCH + 64 * (i & 1) + 16 * qq) = uint2{P[qq][0], P[qq][1]};
       }
       };
-      if (i == j && dout) tile(std::true_type{});
+      if (dout && j == i + dshift) tile(std::true_type{});
       else tile(std::false_type{});
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -561,7 +629,13 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
     // load for pending when the next tile begins, and waits for everything in flight in the middle
     // of the main loop.
     if constexpr (has_e) {
-      if (i == 3) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+      if (i == NQ - 1) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+      if constexpr (TRI) {   // the tile the next quarter has and this one had not
+        if (i < NQ - 1) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) ev[i + 1][t] = FM_ET(i + 1, i + 1, t);
+        }
+      }
     }
 
     if (direct) {
@@ -571,12 +645,15 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
 #pragma unroll
         for (int it = 0; it < 4; ++it) d[it] = *reinterpret_cast<const uint4*>(tr + 4 * (4 * half + it) * QT_PITCH);
 #pragma unroll
-        for (int it = 0; it < 4; ++it) buf_store16(c_buf, c_lane, (8 * i + 4 * half + it) * c_row, d[it]);
+        for (int it = 0; it < 4; ++it) {
+          // TRI: columns 0 .. 32 (i + 1) of the quarter only
+          if (!TRI || (lane & 15) < 4 * (i + 1)) buf_store16(c_buf, c_lane, (8 * i + 4 * half + it) * c_row, d[it]);
+        }
       }
     }
     if (mirror && (i & 1)) {   // two quarters of the mirrored copy: 128 columns x 128 bytes
 #pragma unroll
-      for (int grp = 0; grp < 4; ++grp) {
+      for (int grp = 0; grp < (TRI ? i : 4); ++grp) {   // columns 32 grp .. +31
         uint2 d[4][2];
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -585,9 +662,12 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, bool
           d[it][1] = *reinterpret_cast<const uint2*>(src + 8);
         }
 #pragma unroll
-        for (int it = 0; it < 4; ++it)
-          buf_store16(c2_buf, c2_lane, (4 * grp + it) * c2_col + 128 * (i >> 1),
-                      uint4{d[it][0].x, d[it][0].y, d[it][1].x, d[it][1].y});
+        for (int it = 0; it < 4; ++it) {
+          // TRI: a lane's 8 rows lie in quarter i - 1 or i; tile (quarter, grp) is mirrored when grp < quarter
+          if (!TRI || grp < i - 1 + (int)((lane & 7) >> 2))
+            buf_store16(c2_buf, c2_lane, (4 * grp + it) * c2_col + 128 * (i >> 1),
+                        uint4{d[it][0].x, d[it][0].y, d[it][1].x, d[it][1].y});
+        }
       }
     }
   }
@@ -615,6 +695,7 @@ struct FastArgs {
   int tail_slot0;       // first slot of the last round's sub-parts
   int reduce_tile0;     // first tile the second kernel has to finish
   int sub64;            // the left-over tiles are computed whole-k as 64x64 sub-tiles, 16 workgroups each
+  int half;             // the items are 128x256 half tiles, never cut (the NI == 2 kernels)
 };
 
 // k stages [kb, ke) of base part `part` of `parts`, or of its sub-part `sub` of `subs`
@@ -663,6 +744,56 @@ __device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& b, int&
     }
   }
   ti = tj = 0;   // not reached for pos < num_tiles
+}
+
+// Position in the half-tile schedule -> tile and half.  A product that is not symmetric has two
+// items per tile, the upper (h = 0) and the lower 128 rows.  A symmetric one has its diagonal tiles
+// as one item each (`whole_diag`), so a matrix of T x T tiles makes T (T - 1) + T = T^2 items; the
+// order is that of tile_at, the two halves of a tile next to each other.
+__device__ __forceinline__ void half_item_at(const GemmArgs& g, int e, int& b, int& ti, int& tj, int& h, bool& whole_diag) {
+  whole_diag = false;
+  if (!g.symmetric) {
+    h = e & 1;
+    tile_at(g, e >> 1, b, ti, tj);
+    return;
+  }
+  constexpr int SB = 8;
+  b = 0;
+  if (g.batch > 1) {
+    const int per_matrix = g.tiles_m * g.tiles_m;
+    b = e / per_matrix;
+    e -= b * per_matrix;
+  }
+  const int nb = (g.tiles_m + SB - 1) / SB;
+  for (int I = 0; I < nb; ++I) {
+    const int rows = (g.tiles_m - I * SB) < SB ? (g.tiles_m - I * SB) : SB;
+    for (int J = I; J < nb; ++J) {
+      const int cols = (g.tiles_m - J * SB) < SB ? (g.tiles_m - J * SB) : SB;
+      const int cnt = I == J ? rows * rows : 2 * rows * cols;
+      if (e < cnt) {
+        if (I == J) {
+          int a = 0;
+          for (; a < rows - 1; ++a) {            // row a of the triangle: its diagonal tile, then 2 (rows - 1 - a) halves
+            const int in_row = 2 * (rows - a) - 1;
+            if (e < in_row) break;
+            e -= in_row;
+          }
+          ti = I * SB + a;
+          whole_diag = e == 0;
+          tj = whole_diag ? ti : ti + 1 + ((e - 1) >> 1);
+          h = whole_diag ? 0 : (e - 1) & 1;
+        } else {
+          const int t = e >> 1, a = t / cols;
+          h = e & 1;
+          ti = I * SB + a;
+          tj = J * SB + (t - a * cols);
+        }
+        return;
+      }
+      e -= cnt;
+    }
+  }
+  ti = tj = h = 0;   // not reached for e < the number of items
 }
 
 // ---- 64x64 sub-tiles of the tiles left over after the last full round ---------------------------
@@ -805,7 +936,7 @@ __device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, in
 }
 
 // MODE: how whole tiles are written out (see epilogue_regs); chosen by the host from E and beta
-template <bool F16, int MODE>
+template <bool F16, int MODE, int NI>
 __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   // two operand stages (A0 B0 A1 B1, 32 KiB each) during the main loop, the accumulator staging of
   // the four waves afterwards
@@ -826,19 +957,23 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   const uint32_t ldsw = FM_LDS_ADDR(smem) + wave * 1024;   // where this wave's copies land inside a slot
 
   // per-lane fragment addresses (row = lane % 32 of the fragment's 32 rows, k half = lane / 32)
-  FragAddr fa;
+  FragAddr<NI> fa;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int ra = wm * 128 + i * 32 + (lane & 31);
-    const int rb = wn * 128 + i * 32 + (lane & 31);
+  for (int i = 0; i < NI; ++i) {
+    const int ra = wm * (32 * NI) + i * 32 + (lane & 31);
     const uint32_t ao = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
-    const uint32_t bo = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       fa.a_lo[i][ks] = ao ^ (ks << 5);
       fa.a_hi[i][ks] = (ao ^ (ks << 5)) + a_slot_off(2);
-      fa.b[i][ks] = (bo ^ (ks << 5)) + b_slot_off(0);
     }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int rb = wn * 128 + i * 32 + (lane & 31);
+    const uint32_t bo = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) fa.b[i][ks] = (bo ^ (ks << 5)) + b_slot_off(0);
   }
 
   for (int round = 0; round <= p.rounds; ++round) {
@@ -847,7 +982,13 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       item = round * p.grid + w;
       slot_id = item;
       item_range(p.nk, p.ksplit > 1 ? item % p.ksplit : 0, p.ksplit, 0, 1, kb, ke);
-    } else if (p.sub64) {
+    } else if (NI == 2) {   // half tiles are never cut
+      if (w >= p.rem) break;
+      item = p.rounds * p.grid + w;
+      slot_id = 0;
+      kb = 0;
+      ke = p.nk;
+    } else if (NI == 4 && p.sub64) {
       if (w >= p.rem * 16) break;
       int sbi, sti, stj;
       tile_at(p.g, p.rounds * p.grid + (w >> 4), sbi, sti, stj);
@@ -861,52 +1002,112 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       slot_id = p.tail_slot0 + w;
       item_range(p.nk, p.ksplit > 1 ? item % p.ksplit : 0, p.ksplit, sub, p.split, kb, ke);
     }
-    const int pos = p.ksplit > 1 ? item / p.ksplit : item;
     const int n = ke - kb;
-    int bi, ti, tj;
-    tile_at(p.g, pos, bi, ti, tj);
+    int bi, ti, tj, half = 0;
+    bool ditem = false;   // NI == 2: a whole diagonal tile of a symmetric product
+    if constexpr (NI == 2) half_item_at(p.g, item, bi, ti, tj, half, ditem);
+    else tile_at(p.g, p.ksplit > 1 ? item / p.ksplit : item, bi, ti, tj);
     const GemmArgs g = batch_view(p.g, bi);
-    const int m0 = ti * BM, n0 = tj * BN;
+    const int m0 = ti * BM + half * 128, n0 = tj * BN;
 
     // DMA copy q of this wave fills LDS rows (q*4 + wave)*8 .. +8 of an operand stage (the output
     // is a whole number of tiles on this path, so every row exists)
-    uint32_t voA[8], voB[8];
+    uint32_t voA[2 * NI], voB[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int row = (q * 4 + wave) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ swz(row);
-      voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
+      if (q < 2 * NI) voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
       voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
     }
     const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
     const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
 
-    f32x16_t acc[4][4];   // started from zero by the first substep of the first stage
+    f32x16_t acc[NI == 2 ? 3 : 4][4];   // started from zero by the first substep of the first stage
 
+    const bool tri = NI == 2 && ditem && wave < 2;
+    bool looped = false;
+    if constexpr (NI == 2) {
+     if (ditem) {
+      looped = true;
+      // ---- a diagonal tile as one item: its panel (operand B's offsets: A == B) through the A slots ----
+      DFragAddr dfa;
+      int dlane = lane;   // derived anew for every such item instead of being kept across the others
+      asm volatile("" : "+v"(dlane));
+#pragma unroll
+      for (int q = 0; q < 6; ++q) {
+        const int r0 = tri ? 128 * wave + 32 * (q & 3) : (q < 2 ? 64 * (wave - 2) + 32 * q : 128 + 32 * (q - 2));
+        const int r = r0 + (dlane & 31);
+        const uint32_t o = (uint32_t)(r * ROWB + (((dlane >> 5) ^ swz(r)) << 4));
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          dfa.lo[q][ks] = o ^ (ks << 5);
+          dfa.hi[q][ks] = (o ^ (ks << 5)) + a_slot_off(2);
+        }
+      }
+      const int last = n - 1;
+      const int k1 = last < 1 ? last : 1;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, a_slot_off(0) + q * 4096);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
+      wait_vmcnt<8>();
+      __syncthreads();
+      auto dloop = [&](auto tri_tag) {
+        constexpr bool TRI = decltype(tri_tag)::value;
+        DFrag f0, f1;
+#pragma unroll
+        for (int q = 0; q < (TRI ? 4 : 6); ++q) f0.f[q] = read_d<0>(smem, dfa, q, 0);
+#define FM_DSTAGE(AS, S, FIRST)                                                                  \
+        {                                                                                        \
+          const int kn = (S) + 2 < last ? (S) + 2 : last;                                        \
+          dstage<F16, TRI, AS, FIRST>(acc, f0, f1, smem, dfa, voB, gB + kn * BKF, ldsw);         \
+        }
+        FM_DSTAGE(0, 0, true)
+        int s = 1;
+        for (; s + 3 <= n; s += 3) {
+          FM_DSTAGE(1, s, false)
+          FM_DSTAGE(2, s + 1, false)
+          FM_DSTAGE(0, s + 2, false)
+        }
+        if (s < n) {
+          FM_DSTAGE(1, s, false)
+          if (s + 1 < n) FM_DSTAGE(2, s + 1, false)
+        }
+#undef FM_DSTAGE
+      };
+      if (tri) dloop(std::true_type{});
+      else dloop(std::false_type{});
+      wait_vmcnt<0>();
+      __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
+     }
+    }
     // ---- main loop over k stages kb .. ke-1 ----------------------------------------------------
-    {
-      Frag f0, f1;
+    if (!looped) {
+      Frag<NI> f0, f1;
       // stages past the end are the last stage again (into slots nobody reads), so that the number
       // of copies in flight is the same at every wait
       const int last = n - 1;
       const int k1 = last < 1 ? last : 1;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
+      for (int q = 0; q < 2 * NI; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
 #pragma unroll
       for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, b_slot_off(0) + q * 4096);
 #pragma unroll
-      for (int q = 0; q < 8; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
+      for (int q = 0; q < 2 * NI; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
 #pragma unroll
       for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, b_slot_off(1) + q * 4096);
-      wait_vmcnt<16>();
+      wait_vmcnt<2 * NI + 8>();
       __syncthreads();
 #pragma unroll
-      for (int q = 0; q < 4; ++q) { f0.a[q] = read_a<0>(smem, fa, q, 0); f0.b[q] = read_b<0>(smem, fa, q, 0); }
+      for (int q = 0; q < NI; ++q) f0.a[q] = read_a<0>(smem, fa, q, 0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) f0.b[q] = read_b<0>(smem, fa, q, 0);
       // the slots come round every 6 stages; the first stage stands apart
 #define FM_STAGE_T(AS, BS, S, FIRST)                                                             \
       {                                                                                          \
         const int kn = (S) + 2 < last ? (S) + 2 : last;                                          \
-        stage<F16, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
+        stage<F16, NI, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
       }
 #define FM_STAGE(AS, BS, S) FM_STAGE_T(AS, BS, S, false)
       FM_STAGE_T(0, 0, 0, true)
@@ -940,27 +1141,43 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
 
     // ---- write-out -------------------------------------------------------------------------------
     const bool split = (n != p.nk);
-    const bool diag = g.symmetric && ti == tj;
-    const int row0 = m0 + wm * 128, col0 = n0 + wn * 128;
-    unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
-    if (split) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
-      const EpiLds L = epi_lds(wave_lds);
-      float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
-#define FM_QUARTER(q)                                                        \
-      stage_store<q, 4>(acc, L.F, lane);                                     \
-      copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);
-      FM_QUARTER(0)
-      FM_QUARTER(1)
-      FM_QUARTER(2)
-      FM_QUARTER(3)
-#undef FM_QUARTER
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));
-      epilogue_regs<F16, MODE>(g, diag, wm == wn, acc, wave_lds, row0, col0, lane);
+    const bool diag = NI == 4 && g.symmetric && ti == tj;   // (the half tiles of a symmetric product lie off the diagonal)
+    int row0 = m0 + wm * (32 * NI), col0 = n0 + wn * 128;
+    if (NI == 2 && ditem) {   // the squares on the diagonal, or 64 rows of the one above it
+      row0 = tri ? m0 + 128 * wave : m0 + 64 * (wave - 2);
+      col0 = tri ? row0 : m0 + 128;
     }
+    unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
+    // (the accumulators are pinned to their registers first: see the note on element reads above)
+#define FM_WRITE_OUT                                                                             \
+    {                                                                                            \
+      _Pragma("unroll") for (int i = 0; i < NI; ++i)                                             \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));        \
+      epilogue_regs<F16, MODE, NI, false>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane); \
+    }
+    if constexpr (NI == 4) {
+      if (split) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
+        const EpiLds L = epi_lds(wave_lds);
+        float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
+#define FM_QUARTER(q)                                                        \
+        stage_store<q, 4>(acc, L.F, lane);                                     \
+        copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);
+        FM_QUARTER(0)
+        FM_QUARTER(1)
+        FM_QUARTER(2)
+        FM_QUARTER(3)
+#undef FM_QUARTER
+      } else {
+        FM_WRITE_OUT
+      }
+    } else if (tri) {
+#pragma unroll
+      for (int q = 0; q < 10; ++q) asm volatile("" : "+a"(acc[tri_r(tri_i(q), tri_j(q))][tri_c(tri_i(q), tri_j(q))]));
+      epilogue_regs<F16, MODE, NI, true>(g, false, 0, acc, wave_lds, row0, col0, lane);
+    } else {
+      FM_WRITE_OUT
+    }
+#undef FM_WRITE_OUT
     __syncthreads();   // the next tile's copies land in the memory the staging just used
   }
 }
@@ -1145,8 +1362,6 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
   epilogue_quarter<F16>(g, diag, F, e_buf, RA, 0, row0, col0, lane, 0, 8, 3);
 }
 
-inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
-
 }  // namespace
 
 // Too few tiles for one round (M = 4096 gives 136 symmetric tiles) and a long k: every tile is cut
@@ -1226,6 +1441,17 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
   return true;
 }
 
+// The half-tile schedule (128x256 items, a diagonal tile of a symmetric product as one item) is
+// taken when all its items fit into one round: the whole tiles of such a problem would leave about
+// half of the CUs idle, and its items are never cut, so nothing is added up afterwards.  With more
+// items than workgroups whole tiles win: a stage of a half tile costs more than half a stage of a
+// whole one (48 KiB of operands for half the MFMAs).
+static bool half_schedule_chosen(long long half_items, int nk, int grid) {
+  const long long k = knob(kKnobHalf);
+  if (k >= 0) return k > 0;
+  return knob(kKnobKsplit) < 0 && half_items <= grid && nk >= 8;
+}
+
 bool gemm_fast_eligible(const GemmArgs& a) {
   if (!tiled_dma_eligible(a, BM)) return false;
   // the write-out reads the epilogue operand transposed, 16 bytes at a time
@@ -1245,6 +1471,14 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
   const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
   const double t_small = (double)((small_tiles + cus - 1) / cus) * (nk * 0.55 + 6.0);
+  const long long half_items = (a.symmetric ? tm * tm : 2 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
+  if (half_schedule_chosen(half_items, nk, cus)) {
+    // a stage of a half tile takes 0.435 us at the clock of a part-filled chip and up to 0.75 us
+    // when every CU works; the 128x128 tiles keep the benefit of the doubt
+    const double occ = (double)half_items / cus;
+    const double t_half = nk * (0.435 + 0.8 * (occ > 0.6 ? occ - 0.6 : 0.0)) + 18.0;
+    if (t_half < 0.8 * t_small) return true;
+  }
   return t_large < t_small;
 }
 
@@ -1292,18 +1526,43 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   f.nk = a.Kc / BKF;
   const long long have = ws ? (long long)(ws_bytes / (PART_FLOATS * sizeof(float))) : 0;
   fast_schedule(a.num_tiles, f.nk, have < kMaxSlots ? have : kMaxSlots, f);
+  f.half = 0;
+  int grid = cu_count() < kMaxGrid ? cu_count() : kMaxGrid;
+  const long long kg = knob(kKnobGrid);
+  if (kg > 0 && kg < grid) grid = (int)kg;
+  const long long half_items = a.symmetric ? (long long)a.tiles_m * a.tiles_m * a.batch : 2LL * a.num_tiles;   // a diagonal tile is one item
+  if (half_items < (1LL << 30) && half_schedule_chosen(half_items, f.nk, grid)) {   // 128x256 half tiles, whole, in rounds
+    const int items = (int)half_items;
+    if (grid > items) grid = items;
+    f.half = 1;
+    f.grid = grid;
+    f.ksplit = 1;
+    f.rounds = items / grid;
+    f.rem = items % grid;
+    f.split = 1;
+    f.sub64 = 0;
+    f.tail_slot0 = 0;
+    f.reduce_tile0 = a.num_tiles;
+  }
   f.partials = static_cast<float*>(ws);
+  if (f.half) {
+    if (a.elem == kElemF16) hipLaunchKernelGGL((gemm_nt_rounds_kernel<true, 0, 2>), dim3(f.grid), dim3(256), 0, stream, f);
+    else if (!a.E) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 0, 2>), dim3(f.grid), dim3(256), 0, stream, f);
+    else if (a.beta == 1.0f) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 1, 2>), dim3(f.grid), dim3(256), 0, stream, f);
+    else hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 2, 2>), dim3(f.grid), dim3(256), 0, stream, f);
+    return (int)hipGetLastError();
+  }
   const int slots = f.tail_slot0 + f.rem * f.split;
   const int reduce_tiles = a.num_tiles - f.reduce_tile0;
   if (reduce_tiles > 0 && (slots > have || f.ksplit * f.split > kMaxParts)) return kErrWorkspace;
   if (a.elem == kElemF16) {
-    hipLaunchKernelGGL((gemm_nt_rounds_kernel<true, 0>), dim3(f.grid), dim3(256), 0, stream, f);
+    hipLaunchKernelGGL((gemm_nt_rounds_kernel<true, 0, 4>), dim3(f.grid), dim3(256), 0, stream, f);
     if (reduce_tiles > 0)
       hipLaunchKernelGGL(gemm_nt_reduce_kernel<true>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
   } else {
-    if (!a.E) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 0>), dim3(f.grid), dim3(256), 0, stream, f);
-    else if (a.beta == 1.0f) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 1>), dim3(f.grid), dim3(256), 0, stream, f);
-    else hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 2>), dim3(f.grid), dim3(256), 0, stream, f);
+    if (!a.E) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 0, 4>), dim3(f.grid), dim3(256), 0, stream, f);
+    else if (a.beta == 1.0f) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 1, 4>), dim3(f.grid), dim3(256), 0, stream, f);
+    else hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 2, 4>), dim3(f.grid), dim3(256), 0, stream, f);
     if (reduce_tiles > 0)
       hipLaunchKernelGGL(gemm_nt_reduce_kernel<false>, dim3(reduce_tiles * 16), dim3(256), 0, stream, f);
   }

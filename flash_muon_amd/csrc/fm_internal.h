@@ -21,7 +21,7 @@ constexpr int kErrWorkspace = -2;     // the schedule needs more partial-tile sl
 // Tuning knobs (fm_set_knob, include/flashmuon.h); the FLASHMUON_* environment variables of the same
 // names give their initial values, read once when the library is first used.  A negative value
 // means "decide automatically".
-constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobNoSub64 = 4, kKnobCount = 5;
+constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobNoSub64 = 4, kKnobHalf = 5, kKnobCount = 6;
 long long knob(int which);
 int set_knob(int which, long long value);
 // compute units of the current device (queried once per device)

@@ -56,7 +56,7 @@ FM_API const char* fm_version(void);
 
 /* Tuning knobs, for experiments and for tests that have to reach a particular schedule.  A
  * negative value gives the decision back to the library.  The environment variables
- * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS, FLASHMUON_NO_MID and FLASHMUON_NO_SUB64 set the initial
+ * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS, FLASHMUON_NO_MID, FLASHMUON_NO_SUB64 and FLASHMUON_HALF set the initial
  * values; they are read once, when the library is first used, never per call.  No counterpart in
  * the reference (its tuning is Triton's autotune table, flash_muon/matmul_transpose_triton.py:6-18).
  */
@@ -65,8 +65,10 @@ enum fm_knob {
   FM_KNOB_KSPLIT = 1,          /* base parts every tile of that schedule is cut into along k */
   FM_KNOB_FAST_MIN_UNITS = 2,  /* take the 256x256 schedule when tiles * k-stages >= this (0: whenever the shape allows) */
   FM_KNOB_NO_MID = 3,          /* 1: never take the 128x128 copy-fed schedule */
-  FM_KNOB_NO_SUB64 = 4         /* 1: cut the tiles left after the last full round along k (fp32 parts, second
+  FM_KNOB_NO_SUB64 = 4,        /* 1: cut the tiles left after the last full round along k (fp32 parts, second
                                   kernel) even where 64x64 sub-tiles over the whole k would do */
+  FM_KNOB_HALF = 5             /* 1: always, 0: never run the 256x256 schedule on 128x256 half tiles (taken by
+                                  itself when all of them fit into one round of workgroups) */
 };
 FM_API int fm_set_knob(int knob, long long value);
 

@@ -15,6 +15,7 @@ DEV = "cuda:0"
 @pytest.fixture(autouse=True)
 def _small_inputs_take_the_256_path(knobs):
     knobs("FLASHMUON_FAST_MIN_UNITS", 0)
+    knobs("FLASHMUON_HALF", 0)   # whole tiles: the half-tile schedule has tests of its own
 
 
 def _ints(shape, seed, lo=-2, hi=2):
