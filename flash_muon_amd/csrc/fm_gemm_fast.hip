@@ -147,13 +147,15 @@ __device__ __forceinline__ void stage(f32x16_t (&acc)[NR][4], Frag<NI>& f0, Frag
 
 // ---- a diagonal tile of a symmetric product as one item of the half-tile schedule ---------------
 // Of the 8 x 8 MFMA tiles of a diagonal 256x256 tile only those on or below the diagonal are
-// distinct: 36, against the 32 of a half tile.  They are shared out 10, 10, 8, 8: waves 0 and 1
-// take the lower triangles of the two 128x128 squares on the diagonal (4 fragments, 10 MFMAs per
-// substep), waves 2 and 3 a 64x128 half each of the square above the diagonal, in the shape of any
-// other wave of the half-tile kernel.  Both operands are the one 256-row panel, which goes round
-// the three A slots (8 copies per wave and stage, issued two stages ahead); the B slots are idle.
-struct DFrag { bf16x8_t f[6]; };   // triangle waves: rows 32q of their square; the others: 2 row and 4 column fragments
-struct DFragAddr { uint32_t lo[6][4], hi[6][4]; };   // A slots 0 and 1 / A slot 2
+// distinct: 36, against the 32 of a half tile, 9 per wave.  Waves 0 and 1 take the lower triangles
+// of the two 128x128 squares on the diagonal, without tile (1, 0) (4 fragments, 9 MFMAs per
+// substep); waves 2 and 3 a 64x128 half each of the square above the diagonal, in the shape of any
+// other wave of the half-tile kernel, and tile (1, 0) of the first and the second square (two more
+// fragments, read once more rather than picked from the six at the cost of vector instructions
+// among the MFMAs).  Both operands are the one 256-row panel, which goes round the three A slots
+// (8 copies per wave and stage, issued two stages ahead); the B slots are idle.
+struct DFrag { bf16x8_t f[8]; };   // triangle waves: rows 32q of their square; the others: 2 row, 4 column fragments and the ninth tile's two
+struct DFragAddr { uint32_t lo[8][4], hi[8][4]; };   // A slots 0 and 1 / A slot 2
 
 template <int ASLOT>
 __device__ __forceinline__ bf16x8_t read_d(const unsigned char* smem, const DFragAddr& fa, int q, int ks) {
@@ -164,18 +166,18 @@ __device__ __forceinline__ bf16x8_t read_d(const unsigned char* smem, const DFra
 // where a triangle wave keeps MFMA tile (i, j), j <= i, among its 3 x 4 accumulator tuples
 __host__ __device__ constexpr int tri_r(int i, int j) { return i < 3 ? i : (j < 3 ? 0 : 1); }
 __host__ __device__ constexpr int tri_c(int i, int j) { return i < 3 ? j : (j < 3 ? j + 1 : 2); }
-// row and column fragment of MFMA q of a triangle wave, in the order (0,0) (1,0) (1,1) (2,0) ...
-__host__ __device__ constexpr int tri_i(int q) { return q < 1 ? 0 : q < 3 ? 1 : q < 6 ? 2 : 3; }
-__host__ __device__ constexpr int tri_j(int q) { return q - tri_i(q) * (tri_i(q) + 1) / 2; }
+// row and column fragment of MFMA q of a triangle wave: (0,0) (1,1) (2,0) (2,1) (2,2) (3,0) .. (3,3)
+__host__ __device__ constexpr int tri_i(int q) { return q < 2 ? q : q < 5 ? 2 : 3; }
+__host__ __device__ constexpr int tri_j(int q) { return q < 2 ? q : q < 5 ? q - 2 : q - 5; }
 
-// the MFMAs of one substep: 10 (TRI) or 8, with READS fragment reads of `ks_next` of slot RSLOT
-// riding on the first ones and copies Q0 .. Q1-1 of the panel two stages ahead on the later ones
+// the 9 MFMAs of one substep, with the fragment reads of `ks_next` of slot RSLOT riding on the
+// first ones and copies Q0 .. Q1-1 of the panel two stages ahead on the later ones.
 template <bool F16, bool TRI, int RSLOT, int Q0, int Q1, int CSLOT, bool FIRST>
 __device__ __forceinline__ void dsubstep(f32x16_t (&acc)[3][4], const DFrag& cur, DFrag& nxt, const unsigned char* smem,
                                          const DFragAddr& fa, int ks_next, const uint32_t (&vo)[8], const bf16_t* gP,
                                          uint32_t ldsw) {
-  constexpr int NM = TRI ? 10 : 8, NRD = TRI ? 4 : 6;
-  constexpr int C0 = 5, CSTEP = TRI ? 2 : 1;   // copies after MFMA 5, 7, 9 or 5, 6, 7
+  constexpr int NM = 9, NRD = TRI ? 4 : 8;
+  constexpr int C0 = 5, CSTEP = 1;   // copies after MFMA 5, 6, 7
 #pragma unroll
   for (int q = 0; q < NM; ++q) {
     if (q < NRD) nxt.f[q] = read_d<RSLOT>(smem, fa, q, ks_next);
@@ -185,9 +187,11 @@ __device__ __forceinline__ void dsubstep(f32x16_t (&acc)[3][4], const DFrag& cur
     if constexpr (TRI) {
       f32x16_t& c = acc[tri_r(tri_i(q), tri_j(q))][tri_c(tri_i(q), tri_j(q))];
       c = mfma_32x32x16<F16>(cur.f[tri_i(q)], cur.f[tri_j(q)], FIRST ? zero : c);
-    } else {
+    } else if (q < 8) {
       f32x16_t& c = acc[q >> 2][q & 3];
       c = mfma_32x32x16<F16>(cur.f[q >> 2], cur.f[2 + (q & 3)], FIRST ? zero : c);
+    } else {   // tile (1, 0) of a diagonal square: rows 32 .. 63 times rows 0 .. 31 of it
+      acc[2][0] = mfma_32x32x16<F16>(cur.f[6], cur.f[7], FIRST ? zero : acc[2][0]);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -492,14 +496,26 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 // The wave's block is 32 NI rows x 128 columns at (row0, col0).  `diag`: the block has no mirror
 // image to write (it lies in a diagonal tile of a symmetric product, which holds both); `dshift`:
 // MFMA tile (i, i + dshift) of the block lies on the diagonal of the output, or a value no tile has.
-// TRI: the block is a 128x128 square on the diagonal of a symmetric product of which the wave
-// holds the MFMA tiles (i, j), j <= i, at acc[tri_r(i, j)][tri_c(i, j)]: those are written in
-// place, and the ones below the diagonal also as their mirror images above it.
-template <bool F16, int MODE, int NI, bool TRI, int NR>
+// KIND 1 and 2: the block is a 128x128 square on the diagonal of a symmetric product, of which the
+// wave holds some MFMA tiles on or below the diagonal (1: all but (1, 0), at
+// acc[tri_r(i, j)][tri_c(i, j)]; 2: (1, 0) alone, at acc[2][0]).  Those are written in place, and
+// the ones below the diagonal also as their mirror images above it.
+__host__ __device__ constexpr bool epi_has(int kind, int i, int j) {
+  return kind == 0 ? true : kind == 1 ? (j <= i && !(i == 1 && j == 0)) : (i == 1 && j == 0);
+}
+__host__ __device__ constexpr bool epi_row_has(int kind, int i) {
+  return i >= 0 && (epi_has(kind, i, 0) || epi_has(kind, i, 1) || epi_has(kind, i, 2) || epi_has(kind, i, 3));
+}
+__host__ __device__ constexpr bool epi_mirrors(int kind, int i, int j) {   // tile (i, j) has a mirror image to write
+  return kind == 0 ? true : (i >= 0 && j < i && epi_has(kind, i, j));
+}
+
+template <bool F16, int MODE, int NI, int KIND, int NR>
 __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int dshift,
                                               const f32x16_t (&acc)[NR][4], unsigned char* T, int row0, int col0,
                                               int lane) {
-  constexpr int NQ = TRI ? 4 : NI;   // quarters: rows of MFMA tiles
+  constexpr bool TRI = KIND != 0;
+  constexpr int NQ = KIND == 0 ? NI : KIND == 1 ? 4 : 2;   // quarters: rows of MFMA tiles
   // what follows is derived from `lane` anew for every tile: kept in registers across the main
   // loop instead, the per-lane offsets of the write-out would crowd out the loop's own
   asm volatile("" : "+v"(lane));
@@ -507,7 +523,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
   const int lc = lane & 31, lh = lane >> 5, par = lane & 1;
   const bool direct = g.C != nullptr;
   const bool mirror = g.C2 != nullptr && !diag;
-  const bool dout = (TRI || diag) && g.diag_out != nullptr;
+  const bool dout = (KIND == 1 || (KIND == 0 && diag)) && g.diag_out != nullptr;
   const float alpha = g.alpha, beta = g.beta;
   const uint32_t sel = par ? 0x03020706u : 0x05040100u;   // odd lanes keep the high halves, even lanes the low ones
   float* const RA = reinterpret_cast<float*>(T + QT_BYTES);
@@ -540,9 +556,10 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
       *reinterpret_cast<float2*>(RA + lane * 2) = ra;
     }
 #pragma unroll
-    for (int j = 0; j < (TRI ? 1 : 4); ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int t = 0; t < 2; ++t) ev[j][t] = FM_ET(0, j, t);
+      for (int t = 0; t < 2; ++t)
+        if (epi_has(KIND, 0, j)) ev[j][t] = FM_ET(0, j, t);
   }
 
 #pragma unroll
@@ -557,7 +574,8 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
       }
     }
 #pragma unroll
-    for (int j = 0; j < (TRI ? i + 1 : 4); ++j) {
+    for (int j = 0; j < 4; ++j) {
+      if (!epi_has(KIND, i, j)) continue;
       // the scheduler works on one MFMA tile at a time: left alone with the whole unrolled
       // write-out, it moves every accumulator to a vector register first and runs out of them
       __builtin_amdgcn_sched_barrier(0);
@@ -567,7 +585,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
       constexpr bool DOUT = decltype(dout_tag)::value;
       float v[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) v[r] = acc[TRI ? tri_r(i, j) : i][TRI ? tri_c(i, j) : j][r];
+      for (int r = 0; r < 16; ++r) v[r] = acc[KIND == 0 ? i : KIND == 1 ? tri_r(i, j) : 2][KIND == 0 ? j : KIND == 1 ? tri_c(i, j) : 0][r];
       if constexpr (has_e) {
         uint32_t eb[4][2];   // [qq][h]: the operand in the accumulators' layout
 #pragma unroll
@@ -576,7 +594,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
           swap32(a0, b0);
           swap32(a1, b1);
           eb[2 * t][0] = a0; eb[2 * t][1] = a1; eb[2 * t + 1][0] = b0; eb[2 * t + 1][1] = b1;
-          if (i < NQ - 1) ev[j][t] = FM_ET(i + 1, j, t);
+          if (i < NQ - 1 && epi_has(KIND, i + 1, j)) ev[j][t] = FM_ET(i + 1, j, t);
         }
         if constexpr (MODE == 2) {
 #pragma unroll
@@ -614,7 +632,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
             *reinterpret_cast<uint32_t*>(tw + (8 * qq + 2 * h) * QT_PITCH + 64 * j) = __builtin_amdgcn_perm(nbr, own, sel);
           }
       }
-      if (mirror && (!TRI || j < i)) {   // rows 32(i % 2) + 8qq + 4lh .. +3 of column 32j + lc, for the pass after every second quarter
+      if (mirror && epi_mirrors(KIND, i, j)) {   // rows 32(i % 2) + 8qq + 4lh .. +3 of column 32j + lc, for the pass after every second quarter
 #pragma unroll
         for (int qq = 0; qq < 4; ++qq)
           *reinterpret_cast<uint2*>(mw + 32 * j * QM_PITCH + 64 * (i & 1) + 16 * qq) = uint2{P[qq][0], P[qq][1]};
@@ -630,15 +648,21 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
     // of the main loop.
     if constexpr (has_e) {
       if (i == NQ - 1) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-      if constexpr (TRI) {   // the tile the next quarter has and this one had not
+      if constexpr (TRI) {   // the tiles the next quarter has and this one had not
         if (i < NQ - 1) {
 #pragma unroll
-          for (int t = 0; t < 2; ++t) ev[i + 1][t] = FM_ET(i + 1, i + 1, t);
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+              if (epi_has(KIND, i + 1, j) && !epi_has(KIND, i, j)) ev[j][t] = FM_ET(i + 1, j, t);
         }
       }
     }
 
-    if (direct) {
+    if (direct && epi_row_has(KIND, i)) {
+      // the quarter's columns 32j .. +31 are there when the wave holds tile (i, j)
+      const int cols_there = (epi_has(KIND, i, 0) ? 1 : 0) | (epi_has(KIND, i, 1) ? 2 : 0) |
+                                 (epi_has(KIND, i, 2) ? 4 : 0) | (epi_has(KIND, i, 3) ? 8 : 0);
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         uint4 d[4];
@@ -646,14 +670,14 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
         for (int it = 0; it < 4; ++it) d[it] = *reinterpret_cast<const uint4*>(tr + 4 * (4 * half + it) * QT_PITCH);
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          // TRI: columns 0 .. 32 (i + 1) of the quarter only
-          if (!TRI || (lane & 15) < 4 * (i + 1)) buf_store16(c_buf, c_lane, (8 * i + 4 * half + it) * c_row, d[it]);
+          if (!TRI || ((cols_there >> ((lane & 15) >> 2)) & 1)) buf_store16(c_buf, c_lane, (8 * i + 4 * half + it) * c_row, d[it]);
         }
       }
     }
     if (mirror && (i & 1)) {   // two quarters of the mirrored copy: 128 columns x 128 bytes
 #pragma unroll
-      for (int grp = 0; grp < (TRI ? i : 4); ++grp) {   // columns 32 grp .. +31
+      for (int grp = 0; grp < 4; ++grp) {   // columns 32 grp .. +31: tiles (i - 1, grp) and (i, grp)
+        if (!epi_mirrors(KIND, i - 1, grp) && !epi_mirrors(KIND, i, grp)) continue;
         uint2 d[4][2];
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -663,8 +687,8 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
         }
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
-          // TRI: a lane's 8 rows lie in quarter i - 1 or i; tile (quarter, grp) is mirrored when grp < quarter
-          if (!TRI || grp < i - 1 + (int)((lane & 7) >> 2))
+          // a lane's 8 rows lie in quarter i - 1 or i
+          if (!TRI || ((lane & 7) < 4 ? epi_mirrors(KIND, i - 1, grp) : epi_mirrors(KIND, i, grp)))
             buf_store16(c2_buf, c2_lane, (4 * grp + it) * c2_col + 128 * (i >> 1),
                         uint4{d[it][0].x, d[it][0].y, d[it][1].x, d[it][1].y});
         }
@@ -794,6 +818,90 @@ __device__ __forceinline__ void half_item_at(const GemmArgs& g, int e, int& b, i
     }
   }
   ti = tj = h = 0;   // not reached for e < the number of items
+}
+
+// The k loop of a diagonal item for one kind of wave; the copies of the first two stages are in
+// flight and stage 0 has landed everywhere.
+template <bool F16, bool TRI>
+__device__ __forceinline__ void diag_item_loop(f32x16_t (&acc)[3][4], const unsigned char* smem, const DFragAddr& dfa,
+                                               const uint32_t (&vo)[8], const bf16_t* gP, int n, uint32_t ldsw) {
+  const int last = n - 1;
+  DFrag f0, f1;
+#pragma unroll
+  for (int q = 0; q < (TRI ? 4 : 8); ++q) f0.f[q] = read_d<0>(smem, dfa, q, 0);
+  // stages past the end are the last stage again (into slots nobody reads), so that the number of
+  // copies in flight is the same at every wait
+#define FM_DSTAGE(AS, S, FIRST)                                                                \
+  {                                                                                            \
+    const int kn = (S) + 2 < last ? (S) + 2 : last;                                            \
+    dstage<F16, TRI, AS, FIRST>(acc, f0, f1, smem, dfa, vo, gP + kn * BKF, ldsw);              \
+  }
+  FM_DSTAGE(0, 0, true)
+  int s = 1;
+  for (; s + 3 <= n; s += 3) {
+    FM_DSTAGE(1, s, false)
+    FM_DSTAGE(2, s + 1, false)
+    FM_DSTAGE(0, s + 2, false)
+  }
+  if (s < n) {
+    FM_DSTAGE(1, s, false)
+    if (s + 1 < n) FM_DSTAGE(2, s + 1, false)
+  }
+#undef FM_DSTAGE
+  wait_vmcnt<0>();
+  __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
+}
+
+// A diagonal tile (at m0 on the diagonal) of a symmetric product, over n k stages from gP on.
+template <bool F16, int MODE>
+__device__ __forceinline__ void diag_item(const GemmArgs& g, int m0, int n, unsigned char* smem, const uint32_t (&vo)[8],
+                                          const bf16_t* gP, uint32_t ldsw, int lane, int wave) {
+  const bool tri = wave < 2;
+  DFragAddr dfa;
+  int dlane = lane;   // derived anew for every such item instead of being kept across the others
+  asm volatile("" : "+v"(dlane));
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    // waves 2 and 3: rows 64 (wave - 2) + 32q, columns 128 + 32 (q - 2), and rows 32 .. 63 and 0 .. 31 of square wave - 2
+    const int r0 = tri ? 128 * wave + 32 * (q & 3)
+                       : (q < 2 ? 64 * (wave - 2) + 32 * q : q < 6 ? 128 + 32 * (q - 2) : 128 * (wave - 2) + 32 * (7 - q));
+    const int r = r0 + (dlane & 31);
+    const uint32_t o = (uint32_t)(r * ROWB + (((dlane >> 5) ^ swz(r)) << 4));
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      dfa.lo[q][ks] = o ^ (ks << 5);
+      dfa.hi[q][ks] = (o ^ (ks << 5)) + a_slot_off(2);
+    }
+  }
+  const int k1 = n - 1 < 1 ? n - 1 : 1;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) dma16o(vo[q], gP, ldsw, a_slot_off(0) + q * 4096);
+#pragma unroll
+  for (int q = 0; q < 8; ++q) dma16o(vo[q], gP + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
+  wait_vmcnt<8>();
+  __syncthreads();
+  unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
+  // (each kind of wave has accumulators of its own, pinned to their registers before the write-out)
+  if (tri) {
+    f32x16_t acc[3][4];
+    diag_item_loop<F16, true>(acc, smem, dfa, vo, gP, n, ldsw);
+#pragma unroll
+    for (int q = 0; q < 9; ++q) asm volatile("" : "+a"(acc[tri_r(tri_i(q), tri_j(q))][tri_c(tri_i(q), tri_j(q))]));
+    const int sq = m0 + 128 * wave;
+    epilogue_regs<F16, MODE, 2, 1>(g, false, 0, acc, wave_lds, sq, sq, lane);
+  } else {
+    f32x16_t acc[3][4];
+    diag_item_loop<F16, false>(acc, smem, dfa, vo, gP, n, ldsw);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));
+    asm volatile("" : "+a"(acc[2][0]));
+    // 64 rows of the square above the diagonal, then tile (1, 0) of the first or second square on it
+    epilogue_regs<F16, MODE, 2, 0>(g, false, 0, acc, wave_lds, m0 + 64 * (wave - 2), m0 + 128, lane);
+    const int sq = m0 + 128 * (wave - 2);
+    epilogue_regs<F16, MODE, 2, 2>(g, false, 0, acc, wave_lds, sq, sq, lane);
+  }
 }
 
 // ---- 64x64 sub-tiles of the tiles left over after the last full round ---------------------------
@@ -1023,67 +1131,18 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
     const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
 
-    f32x16_t acc[NI == 2 ? 3 : 4][4];   // started from zero by the first substep of the first stage
-
-    const bool tri = NI == 2 && ditem && wave < 2;
-    bool looped = false;
     if constexpr (NI == 2) {
-     if (ditem) {
-      looped = true;
-      // ---- a diagonal tile as one item: its panel (operand B's offsets: A == B) through the A slots ----
-      DFragAddr dfa;
-      int dlane = lane;   // derived anew for every such item instead of being kept across the others
-      asm volatile("" : "+v"(dlane));
-#pragma unroll
-      for (int q = 0; q < 6; ++q) {
-        const int r0 = tri ? 128 * wave + 32 * (q & 3) : (q < 2 ? 64 * (wave - 2) + 32 * q : 128 + 32 * (q - 2));
-        const int r = r0 + (dlane & 31);
-        const uint32_t o = (uint32_t)(r * ROWB + (((dlane >> 5) ^ swz(r)) << 4));
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          dfa.lo[q][ks] = o ^ (ks << 5);
-          dfa.hi[q][ks] = (o ^ (ks << 5)) + a_slot_off(2);
-        }
+      if (ditem) {   // a diagonal tile of a symmetric product: its panel is operand B's (A == B)
+        diag_item<F16, MODE>(g, m0, n, smem, voB, gB, ldsw, lane, wave);
+        __syncthreads();   // the next item's copies land in the memory the staging just used
+        continue;
       }
-      const int last = n - 1;
-      const int k1 = last < 1 ? last : 1;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, a_slot_off(0) + q * 4096);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
-      wait_vmcnt<8>();
-      __syncthreads();
-      auto dloop = [&](auto tri_tag) {
-        constexpr bool TRI = decltype(tri_tag)::value;
-        DFrag f0, f1;
-#pragma unroll
-        for (int q = 0; q < (TRI ? 4 : 6); ++q) f0.f[q] = read_d<0>(smem, dfa, q, 0);
-#define FM_DSTAGE(AS, S, FIRST)                                                                  \
-        {                                                                                        \
-          const int kn = (S) + 2 < last ? (S) + 2 : last;                                        \
-          dstage<F16, TRI, AS, FIRST>(acc, f0, f1, smem, dfa, voB, gB + kn * BKF, ldsw);         \
-        }
-        FM_DSTAGE(0, 0, true)
-        int s = 1;
-        for (; s + 3 <= n; s += 3) {
-          FM_DSTAGE(1, s, false)
-          FM_DSTAGE(2, s + 1, false)
-          FM_DSTAGE(0, s + 2, false)
-        }
-        if (s < n) {
-          FM_DSTAGE(1, s, false)
-          if (s + 1 < n) FM_DSTAGE(2, s + 1, false)
-        }
-#undef FM_DSTAGE
-      };
-      if (tri) dloop(std::true_type{});
-      else dloop(std::false_type{});
-      wait_vmcnt<0>();
-      __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
-     }
     }
+
+    f32x16_t acc[NI][4];   // started from zero by the first substep of the first stage
+
     // ---- main loop over k stages kb .. ke-1 ----------------------------------------------------
-    if (!looped) {
+    {
       Frag<NI> f0, f1;
       // stages past the end are the last stage again (into slots nobody reads), so that the number
       // of copies in flight is the same at every wait
@@ -1142,18 +1201,14 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     // ---- write-out -------------------------------------------------------------------------------
     const bool split = (n != p.nk);
     const bool diag = NI == 4 && g.symmetric && ti == tj;   // (the half tiles of a symmetric product lie off the diagonal)
-    int row0 = m0 + wm * (32 * NI), col0 = n0 + wn * 128;
-    if (NI == 2 && ditem) {   // the squares on the diagonal, or 64 rows of the one above it
-      row0 = tri ? m0 + 128 * wave : m0 + 64 * (wave - 2);
-      col0 = tri ? row0 : m0 + 128;
-    }
+    const int row0 = m0 + wm * (32 * NI), col0 = n0 + wn * 128;
     unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
     // (the accumulators are pinned to their registers first: see the note on element reads above)
 #define FM_WRITE_OUT                                                                             \
     {                                                                                            \
       _Pragma("unroll") for (int i = 0; i < NI; ++i)                                             \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));        \
-      epilogue_regs<F16, MODE, NI, false>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane); \
+      epilogue_regs<F16, MODE, NI, 0>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane); \
     }
     if constexpr (NI == 4) {
       if (split) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
@@ -1170,10 +1225,6 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       } else {
         FM_WRITE_OUT
       }
-    } else if (tri) {
-#pragma unroll
-      for (int q = 0; q < 10; ++q) asm volatile("" : "+a"(acc[tri_r(tri_i(q), tri_j(q))][tri_c(tri_i(q), tri_j(q))]));
-      epilogue_regs<F16, MODE, NI, true>(g, false, 0, acc, wave_lds, row0, col0, lane);
     } else {
       FM_WRITE_OUT
     }
