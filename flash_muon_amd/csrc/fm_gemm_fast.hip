@@ -1528,7 +1528,7 @@ bool gemm_fast_eligible(const GemmArgs& a) {
     // when every CU works; the 128x128 tiles keep the benefit of the doubt
     const double occ = (double)half_items / cus;
     const double t_half = nk * (0.435 + 0.8 * (occ > 0.6 ? occ - 0.6 : 0.0)) + 18.0;
-    if (t_half < 0.8 * t_small) return true;
+    if (t_half < 0.9 * t_small) return true;
   }
   return t_large < t_small;
 }
