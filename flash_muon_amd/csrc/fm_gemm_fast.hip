@@ -1492,15 +1492,33 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
   return true;
 }
 
+// Estimates in microseconds, from measured costs of a k stage and of a tile's start and write-out.
+// The clock the power cap allows falls as the chip fills, so a stage costs more the more CUs work.
+// One round of whole tiles (cut along k into `ksplit` parts, which adds the fp32 parts and the
+// second kernel):
+static double estimate_whole_round(long long tiles, int nk, int ksplit, int grid) {
+  double occ = (double)(tiles * ksplit) / grid;
+  if (occ > 1.0) occ = 1.0;
+  return (nk / ksplit) * (0.35 + 1.1 * occ) + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
+}
+// one round of half tiles:
+static double estimate_half_round(long long half_items, int nk, int grid) {
+  const double occ = (double)half_items / grid;
+  return nk * (0.50 + 0.78 * (occ > 0.6 ? occ - 0.6 : 0.0)) + 13.0;
+}
+
 // The half-tile schedule (128x256 items, a diagonal tile of a symmetric product as one item) is
-// taken when all its items fit into one round: the whole tiles of such a problem would leave about
-// half of the CUs idle, and its items are never cut, so nothing is added up afterwards.  With more
-// items than workgroups whole tiles win: a stage of a half tile costs more than half a stage of a
-// whole one (48 KiB of operands for half the MFMAs).
-static bool half_schedule_chosen(long long half_items, int nk, int grid) {
+// taken when all its items fit into one round and that round is estimated to be shorter than the
+// round of whole tiles: those would leave about half of the CUs idle, and half items are never
+// cut, so nothing is added up afterwards.  Few tiles with a very long k are better cut along k
+// (16 half items of 1024 stages against 160 parts of 64), and with more items than workgroups
+// whole tiles win: a stage of a half tile costs more than half a stage of a whole one (48 KiB of
+// operands for half the MFMAs).
+static bool half_schedule_chosen(long long half_items, long long tiles, int nk, int grid) {
   const long long k = knob(kKnobHalf);
   if (k >= 0) return k > 0;
-  return knob(kKnobKsplit) < 0 && half_items <= grid && nk >= 8;
+  if (knob(kKnobKsplit) >= 0 || half_items > grid || tiles > grid || nk < 8) return false;
+  return estimate_half_round(half_items, nk, grid) < estimate_whole_round(tiles, nk, auto_ksplit(tiles, nk, grid), grid);
 }
 
 bool gemm_fast_eligible(const GemmArgs& a) {
@@ -1523,13 +1541,8 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
   const double t_small = (double)((small_tiles + cus - 1) / cus) * (nk * 0.55 + 6.0);
   const long long half_items = (a.symmetric ? tm * tm : 2 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
-  if (half_schedule_chosen(half_items, nk, cus)) {
-    // a stage of a half tile takes 0.435 us at the clock of a part-filled chip and up to 0.75 us
-    // when every CU works; the 128x128 tiles keep the benefit of the doubt
-    const double occ = (double)half_items / cus;
-    const double t_half = nk * (0.435 + 0.8 * (occ > 0.6 ? occ - 0.6 : 0.0)) + 18.0;
-    if (t_half < 0.9 * t_small) return true;
-  }
+  // (the 128x128 tiles keep the benefit of the doubt against half tiles)
+  if (half_schedule_chosen(half_items, tiles, nk, cus) && estimate_half_round(half_items, nk, cus) < 0.9 * t_small) return true;
   return t_large < t_small;
 }
 
@@ -1582,7 +1595,7 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   const long long kg = knob(kKnobGrid);
   if (kg > 0 && kg < grid) grid = (int)kg;
   const long long half_items = a.symmetric ? (long long)a.tiles_m * a.tiles_m * a.batch : 2LL * a.num_tiles;   // a diagonal tile is one item
-  if (half_items < (1LL << 30) && half_schedule_chosen(half_items, f.nk, grid)) {   // 128x256 half tiles, whole, in rounds
+  if (half_items < (1LL << 30) && half_schedule_chosen(half_items, a.num_tiles, f.nk, grid)) {   // 128x256 half tiles, whole, in rounds
     const int items = (int)half_items;
     if (grid > items) grid = items;
     f.half = 1;
