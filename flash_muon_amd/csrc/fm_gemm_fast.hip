@@ -268,6 +268,17 @@ __device__ __forceinline__ void stage_store(const f32x16_t (&acc)[NI][4], float*
   }
 }
 
+// one MFMA tile of the accumulators -> columns 32 ct .. +31 of a staged quarter (as stage_store)
+__device__ __forceinline__ void stage_tile(const f32x16_t& a, float* F, int ct, int lane) {
+  const int col = 32 * ct + (lane & 31), rg = 4 * (lane >> 5);
+  float* const dst = F + col * QF_PITCH;
+  const int x = ((col >> 3) & 7) << 2;
+  *reinterpret_cast<f32x4_t*>(dst + ((0 + rg) ^ x)) = __builtin_shufflevector(a, a, 0, 1, 2, 3);
+  *reinterpret_cast<f32x4_t*>(dst + ((8 + rg) ^ x)) = __builtin_shufflevector(a, a, 4, 5, 6, 7);
+  *reinterpret_cast<f32x4_t*>(dst + ((16 + rg) ^ x)) = __builtin_shufflevector(a, a, 8, 9, 10, 11);
+  *reinterpret_cast<f32x4_t*>(dst + ((24 + rg) ^ x)) = __builtin_shufflevector(a, a, 12, 13, 14, 15);
+}
+
 // the 128 x 32 floats of the staged quarter, in staging order, to a partial-tile slot (coalesced)
 __device__ __forceinline__ void copy_stage_to_ws(const float* F, float* dst, int lane) {
 #pragma unroll 8
@@ -1342,23 +1353,26 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
     for (int q = 0; q < 4; ++q) dma16(voB[q], gB + stage * BKF, base + MID_OPER + q * 4096);
   };
 
-  // fragment offsets inside an operand stage (row = lane % 32, k half = lane / 32)
-  uint32_t ao, bo[4];
-  {
-    const int r = wave * 32 + (lane & 31);
-    ao = (uint32_t)(r * ROWB + (((lane >> 5) ^ swz(r)) << 4));
+  // The waves take 64x64 each (2x2 MFMA tiles): 4 fragment reads for 4 MFMAs per substep instead
+  // of the 5 of a 32x128 strip; the loop is bound by the LDS (reads and incoming copies).
+  // Fragment offsets inside an operand stage (row = lane % 32, k half = lane / 32):
+  const int wm = wave >> 1, wn = wave & 1;
+  uint32_t ao[2], bo[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int rb = j * 32 + (lane & 31);
-      bo[j] = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
-    }
+  for (int i = 0; i < 2; ++i) {
+    const int r = wm * 64 + i * 32 + (lane & 31);
+    ao[i] = (uint32_t)(r * ROWB + (((lane >> 5) ^ swz(r)) << 4));
+    const int rb = wn * 64 + i * 32 + (lane & 31);
+    bo[i] = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
   }
 
-  f32x16_t acc[1][4];
+  f32x16_t acc[2][2];
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[0][j][r] = 0.0f;
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   // Stages past the end are the last stage again (into a slot nobody reads), so that the number of
   // copies in flight is the same at every wait.
@@ -1373,30 +1387,37 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
     }
     const unsigned char* sa = smem + (s & (MID_STAGES - 1)) * MID_STAGE;
     const unsigned char* sb = sa + MID_OPER;
-    // the 5 fragment reads of substep ks+1 ride on the 4 MFMAs of substep ks
-    bf16x8_t fa[2], fb[2][4];
-    fa[0] = *reinterpret_cast<const bf16x8_t*>(sa + ao);
+    // the 4 fragment reads of substep ks+1 ride on the 4 MFMAs of substep ks
+    bf16x8_t fa[2][2], fb[2][2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) fb[0][j] = *reinterpret_cast<const bf16x8_t*>(sb + bo[j]);
+    for (int i = 0; i < 2; ++i) {
+      fa[0][i] = *reinterpret_cast<const bf16x8_t*>(sa + ao[i]);
+      fb[0][i] = *reinterpret_cast<const bf16x8_t*>(sb + bo[i]);
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int cur = ks & 1, nxt = cur ^ 1;
       if (ks < 3) {
-        fa[nxt] = *reinterpret_cast<const bf16x8_t*>(sa + (ao ^ ((ks + 1) << 5)));
 #pragma unroll
-        for (int j = 0; j < 4; ++j) fb[nxt][j] = *reinterpret_cast<const bf16x8_t*>(sb + (bo[j] ^ ((ks + 1) << 5)));
+        for (int i = 0; i < 2; ++i) {
+          fa[nxt][i] = *reinterpret_cast<const bf16x8_t*>(sa + (ao[i] ^ ((ks + 1) << 5)));
+          fb[nxt][i] = *reinterpret_cast<const bf16x8_t*>(sb + (bo[i] ^ ((ks + 1) << 5)));
+        }
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[0][j] = mfma_32x32x16<F16>(fa[cur], fb[cur][j], acc[0][j]);
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16<F16>(fa[cur][i], fb[cur][j], acc[i][j]);
       if (ks < 3) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1404,11 +1425,17 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
   wait_vmcnt<0>();
   __syncthreads();   // no copy in flight and no wave still reading: the ring is free
 
-  // one quarter per wave: accumulators -> LDS, then out (the staging areas lie in the ring)
-  float* const F = reinterpret_cast<float*>(smem + wave * (QF_FLOATS * 4));
+  // accumulators -> LDS: MFMA tile (i, j) of this wave belongs to quarter 2 wm + i, columns
+  // 64 wn + 32 j; then every wave finishes one quarter (the staging areas lie in the ring)
   float* const RA = reinterpret_cast<float*>(smem + 4 * (QF_FLOATS * 4) + wave * 128);
   if (use_e && lane < 32) RA[lane] = ra;   // zeros when there are no per-row additions
-  stage_store<0, 1>(acc, F, lane);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      stage_tile(acc[i][j], reinterpret_cast<float*>(smem + (2 * wm + i) * (QF_FLOATS * 4)), 2 * wn + j, lane);
+  __syncthreads();
+  float* const F = reinterpret_cast<float*>(smem + wave * (QF_FLOATS * 4));
   const bool diag = g.symmetric && ti == tj;
   epilogue_quarter<F16>(g, diag, F, e_buf, RA, 0, row0, col0, lane, 0, 8, 3);
 }
