@@ -262,7 +262,7 @@ int launch_gemm_nt(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
     const int rc = launch_gemm_fast(a, ws, ws_bytes, stream);
     if (rc != kErrWorkspace) return rc;
   }
-  if (gemm_mid_eligible(a) && knob(kKnobNoMid) <= 0) return launch_gemm_mid(a, stream);
+  if (gemm_mid_eligible(a) && knob(kKnobNoMid) <= 0) return launch_gemm_mid(a, ws, ws_bytes, stream);
   return launch_gemm_general(a, stream);
 }
 

@@ -293,7 +293,7 @@ __device__ __forceinline__ void copy_stage_to_ws(const float* F, float* dst, int
 // order; `parts` points at the quarter inside slot 0; this wave takes the 16-byte units
 // it_begin*64 .. it_end*64.  Loads go out eight parts at a time.
 __device__ __forceinline__ void sum_parts_to_stage(const float* parts, const int* slots, int nparts, float* F,
-                                                   int lane, int it_begin, int it_end) {
+                                                   int lane, int it_begin, int it_end, int slot_floats = PART_FLOATS) {
   for (int it = it_begin; it < it_end; ++it) {
     const int idx = it * 64 + lane;
     f32x4_t v = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -302,7 +302,7 @@ __device__ __forceinline__ void sum_parts_to_stage(const float* parts, const int
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const int tt = (t0 + t < nparts) ? t0 + t : nparts - 1;   // clamped; the value is dropped below
-        x[t] = *reinterpret_cast<const f32x4_t*>(parts + (size_t)slots[tt] * PART_FLOATS + idx * 4);
+        x[t] = *reinterpret_cast<const f32x4_t*>(parts + (size_t)slots[tt] * slot_floats + idx * 4);
       }
 #pragma unroll
       for (int t = 0; t < 8; ++t) if (t0 + t < nparts) v += x[t];
@@ -1305,8 +1305,19 @@ constexpr int MID_STAGE = 2 * MID_OPER;                 // A and B
 constexpr int MID_RING = MID_STAGES * MID_STAGE;        // 131072; reused by the accumulator staging
 constexpr int MID_SMEM = MID_RING + 4 * QE_BYTES;       // + one E buffer per wave = 163840
 
+// Few tiles and a long k (1024 x 4096: 36 tiles of 64 stages for 256 CUs): every tile is cut along k
+// into `ksplit` parts, one workgroup each, which write their 128x128 fp32 sums to slot
+// tile * ksplit + part of `partials`; gemm_nt_mid_reduce_kernel adds them in k order and runs the
+// epilogue.  Workgroups are numbered part-major, so that neighbours work on the same k range of
+// different tiles and share their operand slices in the L2.
+struct MidSplit {
+  int ksplit;        // 1: whole tiles, written out by this kernel
+  float* partials;
+};
+constexpr int MID_PART_FLOATS = MID_T * MID_T;   // one fp32 partial tile: 64 KiB
+
 template <bool F16>
-__global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
+__global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb, MidSplit sp) {
   __shared__ __align__(1024) unsigned char smem[MID_SMEM];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1317,15 +1328,19 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
     const int chunk = (int)gridDim.x >> 3;
     if (w < chunk * 8) w = (w & 7) * chunk + (w >> 3);
   }
+  const int part = sp.ksplit > 1 ? w / gb.num_tiles : 0;
+  const int tile = w - part * gb.num_tiles;
   int bi, ti, tj;
-  tile_at(gb, w, bi, ti, tj);
+  tile_at(gb, tile, bi, ti, tj);
   const GemmArgs g = batch_view(gb, bi);
   const int m0 = ti * MID_T, n0 = tj * MID_T;
-  const int nk = g.Kc / BKF;
+  const int nk_all = g.Kc / BKF;
+  const int kb = sp.ksplit > 1 ? nk_all * part / sp.ksplit : 0;
+  const int nk = (sp.ksplit > 1 ? nk_all * (part + 1) / sp.ksplit : nk_all) - kb;   // stages of this workgroup
   const int row0 = m0 + wave * 32, col0 = n0;
 
   // the epilogue operand and the per-row additions first: they are long there when needed
-  const bool use_e = !F16 && g.E != nullptr;
+  const bool use_e = !F16 && g.E != nullptr && sp.ksplit == 1;
   unsigned char* const e_buf = smem + MID_RING + wave * QE_BYTES;
   float ra = 0.0f;
   if (use_e) {
@@ -1342,8 +1357,8 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
     voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
     voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
   }
-  const bf16_t* gA = g.A + (int64_t)m0 * g.lda;
-  const bf16_t* gB = g.B + (int64_t)n0 * g.ldb;
+  const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
+  const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
   const uint32_t ring = FM_LDS_ADDR(smem) + wave * 1024;
   auto issue = [&](int stage, int slot) {   // 8 copies per wave
     const uint32_t base = ring + slot * MID_STAGE;
@@ -1436,8 +1451,43 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb) {
       stage_tile(acc[i][j], reinterpret_cast<float*>(smem + (2 * wm + i) * (QF_FLOATS * 4)), 2 * wn + j, lane);
   __syncthreads();
   float* const F = reinterpret_cast<float*>(smem + wave * (QF_FLOATS * 4));
+  if (sp.ksplit > 1) {   // a part of a tile: quarter `wave` of its fp32 sums, in staging order
+    copy_stage_to_ws(F, sp.partials + (size_t)(tile * sp.ksplit + part) * MID_PART_FLOATS + wave * QUARTER_FLOATS, lane);
+    return;
+  }
   const bool diag = g.symmetric && ti == tj;
   epilogue_quarter<F16>(g, diag, F, e_buf, RA, 0, row0, col0, lane, 0, 8, 3);
+}
+
+// Second kernel of the cut 128x128 tiles: one workgroup per (tile, quarter).  Its four waves add
+// the quarter's parts in k order, so the bits do not depend on which workgroup finished when, and
+// share the iterations of its epilogue.
+template <bool F16>
+__global__ __launch_bounds__(256) void gemm_nt_mid_reduce_kernel(GemmArgs gb, MidSplit sp) {
+  __shared__ __align__(1024) unsigned char smem[EPI_WAVE_BYTES];
+  __shared__ int s_slot[kMaxParts];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int t = (int)(blockIdx.x >> 2), q = blockIdx.x & 3;
+  int bi, ti, tj;
+  tile_at(gb, t, bi, ti, tj);
+  const GemmArgs g = batch_view(gb, bi);
+  const EpiLds L = epi_lds(smem);
+  const int row0 = ti * MID_T + 32 * q, col0 = tj * MID_T;
+  if (g.E) {
+    epi_dma_e(g, row0, col0, lane, L.e_addr[0], wave * 2, wave * 2 + 2);
+    if (wave == 0 && lane < 32) L.RA[lane] = g.row_alpha ? g.row_alpha[row0 + lane] : 0.0f;
+  }
+  if ((int)threadIdx.x < sp.ksplit) s_slot[threadIdx.x] = t * sp.ksplit + (int)threadIdx.x;
+  __syncthreads();
+  sum_parts_to_stage(sp.partials + q * QUARTER_FLOATS, s_slot, sp.ksplit, L.F, lane, wave * 4, wave * 4 + 4, MID_PART_FLOATS);
+  wait_vmcnt<0>();
+  __syncthreads();
+  const bool diag = g.symmetric && ti == tj;
+  // direct pass, then (after everybody has put its rounded values back) the transposed pass
+  epilogue_quarter<F16>(g, diag, L.F, L.E[0], L.RA, 0, row0, col0, lane, wave * 2, wave * 2 + 2, 1);
+  __syncthreads();
+  epilogue_quarter<F16>(g, diag, L.F, L.E[0], L.RA, 0, row0, col0, lane, wave * 2, wave * 2 + 2, 2);
 }
 
 }  // namespace
@@ -1519,6 +1569,28 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
   return true;
 }
 
+// Parts per 128x128 tile along k: as many as fill the chip, of at least 4 stages each, when the
+// stages saved outweigh the fp32 round trip and the second launch (estimates in microseconds: 0.55
+// per stage, 6 for a tile's start and write-out, 10 more for the detour).
+static int mid_ksplit(long long tiles, int nk, int grid) {
+  const long long k = knob(kKnobKsplit);
+  int s = 1;
+  if (k >= 1) {
+    s = (int)(k > kMaxParts ? kMaxParts : k);
+  } else if (tiles * 2 <= grid && nk >= 16) {
+    s = (int)(grid / tiles);
+    if (s > nk / 4) s = nk / 4;
+    if (s > 16) s = 16;
+    if (s < 2 || nk * 0.55 + 6.0 <= (nk / s) * 0.55 + 16.0) s = 1;
+  }
+  return s > nk ? nk : s;
+}
+static double estimate_mid(long long tiles, int nk, int grid) {
+  const int s = mid_ksplit(tiles, nk, grid);
+  if (s > 1) return (nk / s) * 0.55 + 16.0;
+  return (double)((tiles + grid - 1) / grid) * (nk * 0.55 + 6.0);
+}
+
 // Estimates in microseconds, from measured costs of a k stage and of a tile's start and write-out.
 // The clock the power cap allows falls as the chip fills, so a stage costs more the more CUs work.
 // One round of whole tiles (cut along k into `ksplit` parts, which adds the fp32 parts and the
@@ -1566,7 +1638,7 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   const int ksplit = auto_ksplit(tiles, nk, cus);
   const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
   const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
-  const double t_small = (double)((small_tiles + cus - 1) / cus) * (nk * 0.55 + 6.0);
+  const double t_small = estimate_mid(small_tiles, nk, cus);
   const long long half_items = (a.symmetric ? tm * tm : 2 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
   // (the 128x128 tiles keep the benefit of the doubt against half tiles)
   if (half_schedule_chosen(half_items, tiles, nk, cus) && estimate_half_round(half_items, nk, cus) < 0.9 * t_small) return true;
@@ -1575,19 +1647,36 @@ bool gemm_fast_eligible(const GemmArgs& a) {
 
 bool gemm_mid_eligible(const GemmArgs& a) { return tiled_dma_eligible(a, MID_T); }
 
-int launch_gemm_mid(GemmArgs a, hipStream_t stream) {
+int launch_gemm_mid(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
   a.tiles_m = a.Ma / MID_T;
   a.tiles_n = a.Nb / MID_T;
   if (a.batch < 1) a.batch = 1;
   a.num_tiles = (a.symmetric ? a.tiles_m * (a.tiles_m + 1) / 2 : a.tiles_m * a.tiles_n) * a.batch;
-  if (a.elem == kElemF16) hipLaunchKernelGGL(gemm_nt_mid_kernel<true>, dim3(a.num_tiles), dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL(gemm_nt_mid_kernel<false>, dim3(a.num_tiles), dim3(256), 0, stream, a);
+  MidSplit sp;
+  sp.ksplit = mid_ksplit(a.num_tiles, a.Kc / BKF, cu_count() < kMaxGrid ? cu_count() : kMaxGrid);
+  sp.partials = static_cast<float*>(ws);
+  // without room for the parts the tiles stay whole
+  if (sp.ksplit > 1 && (!ws || (size_t)a.num_tiles * sp.ksplit * MID_PART_FLOATS * sizeof(float) > ws_bytes)) sp.ksplit = 1;
+  const unsigned grid = (unsigned)(a.num_tiles * sp.ksplit);
+  if (a.elem == kElemF16) hipLaunchKernelGGL(gemm_nt_mid_kernel<true>, dim3(grid), dim3(256), 0, stream, a, sp);
+  else hipLaunchKernelGGL(gemm_nt_mid_kernel<false>, dim3(grid), dim3(256), 0, stream, a, sp);
+  if (sp.ksplit > 1) {
+    if (a.elem == kElemF16) hipLaunchKernelGGL(gemm_nt_mid_reduce_kernel<true>, dim3(a.num_tiles * 4), dim3(256), 0, stream, a, sp);
+    else hipLaunchKernelGGL(gemm_nt_mid_reduce_kernel<false>, dim3(a.num_tiles * 4), dim3(256), 0, stream, a, sp);
+  }
   return (int)hipGetLastError();
 }
 
 size_t gemm_fast_workspace_bytes(int Ma, int Nb, int batch) {
-  if (Ma < BM || Nb < BN || Ma % BM != 0 || Nb % BN != 0) return 0;   // never on this path
   if (batch < 1) batch = 1;
+  // the 128x128 path cuts its tiles along k when at most half the CUs would have one: one round of parts
+  size_t mid_need = 0;
+  if (Ma >= MID_T && Nb >= MID_T && Ma % MID_T == 0 && Nb % MID_T == 0) {
+    const long long m = Ma / MID_T, n = Nb / MID_T;
+    const long long fewest = (Ma == Nb ? m * (m + 1) / 2 : m * n) * batch;
+    if (fewest * 2 <= kMaxGrid) mid_need = (size_t)kMaxGrid * MID_PART_FLOATS * sizeof(float);
+  }
+  if (Ma < BM || Nb < BN || Ma % BM != 0 || Nb % BN != 0) return mid_need;   // never on the 256x256 path
   const long long tm = Ma / BM, tn = Nb / BN;
   // a square output may be a symmetric product (fewer tiles) or a general one: take the larger need
   long long need = 0;
@@ -1604,7 +1693,8 @@ size_t gemm_fast_workspace_bytes(int Ma, int Nb, int batch) {
     }
     if (slots > need) need = slots;
   }
-  return (size_t)need * PART_FLOATS * sizeof(float);
+  const size_t fast_need = (size_t)need * PART_FLOATS * sizeof(float);
+  return fast_need > mid_need ? fast_need : mid_need;
 }
 
 int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {

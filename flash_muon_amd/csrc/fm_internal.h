@@ -126,7 +126,7 @@ size_t gemm_fast_workspace_bytes(int Ma, int Nb, int batch);
 // kErrWorkspace when the schedule needs more than ws holds
 int launch_gemm_fast(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
 bool gemm_mid_eligible(const GemmArgs& a);
-int launch_gemm_mid(GemmArgs args, hipStream_t stream);
+int launch_gemm_mid(GemmArgs args, void* ws, size_t ws_bytes, hipStream_t stream);
 
 // up to kMaxBatch device pointers, passed to a kernel by value
 struct PtrList { void* p[kMaxBatch]; };

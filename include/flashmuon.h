@@ -62,7 +62,7 @@ FM_API const char* fm_version(void);
  */
 enum fm_knob {
   FM_KNOB_GRID = 0,            /* workgroups per launch of the 256x256 schedule (at most one per CU) */
-  FM_KNOB_KSPLIT = 1,          /* base parts every tile of that schedule is cut into along k */
+  FM_KNOB_KSPLIT = 1,          /* parts every tile of that schedule, or of the 128x128 one, is cut into along k */
   FM_KNOB_FAST_MIN_UNITS = 2,  /* take the 256x256 schedule when tiles * k-stages >= this (0: whenever the shape allows) */
   FM_KNOB_NO_MID = 3,          /* 1: never take the 128x128 copy-fed schedule */
   FM_KNOB_NO_SUB64 = 4,        /* 1: cut the tiles left after the last full round along k (fp32 parts, second

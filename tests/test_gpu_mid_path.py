@@ -81,3 +81,60 @@ def test_agrees_with_the_general_path_on_gaussian_input(lib, knobs):
         assert torch.equal(Y, Y.T)
         assert float((Y.float() - ref).norm() / ref.norm()) < 3e-3
     assert float((mid.float() - gen.float()).norm() / ref.norm()) < 3e-3
+
+
+@pytest.fixture
+def no_256_path(knobs):
+    knobs("FLASHMUON_FAST_MIN_UNITS", 10 ** 15)   # whatever the shape, not the 256x256 path
+
+
+@pytest.mark.parametrize("ksplit", [2, 3, 5, 16, 64])
+@pytest.mark.parametrize("M,K", [(128, 1024), (384, 640), (640, 2048), (256, 4096)])
+def test_syrk_tiles_cut_along_k(lib, knobs, no_256_path, M, K, ksplit):
+    """Every 128x128 tile cut into `ksplit` parts along k (the KSPLIT knob; more parts than k stages
+    are capped), their fp32 sums added in k order by the second kernel."""
+    knobs("FLASHMUON_KSPLIT", ksplit)
+    X = _ints((M, K), 17 * M + K + ksplit)
+    want = (X.double() @ X.double().T).float().bfloat16()
+    Y = torch.full((M, M), float("nan"), dtype=torch.bfloat16, device=DEV)
+    gpu_util.syrk(lib, X.to(DEV), Y)
+    assert torch.equal(Y.cpu(), want)
+    assert torch.equal(Y, Y.T)
+
+
+@pytest.mark.parametrize("ksplit", [2, 7])
+def test_poly_axpby_and_f16_tiles_cut_along_k(lib, knobs, no_256_path, ksplit):
+    knobs("FLASHMUON_KSPLIT", ksplit)
+    M, K = 512, 1280
+    g = torch.Generator().manual_seed(M + ksplit)
+    A = torch.randint(-1, 2, (M, M), generator=g)
+    A = (torch.triu(A) + torch.triu(A, 1).T).float().bfloat16()
+    Ad = A.double()
+    full = Ad + 2 * (Ad @ Ad)
+    P, d = gpu_util.syrk_poly(lib, A.to(DEV), 1.0, 2.0, split_diag=True)
+    assert torch.equal(d.cpu().double(), torch.diagonal(full))
+    assert torch.equal(P.cpu(), (full - torch.diag(torch.diagonal(full))).float().bfloat16())
+    X = _ints((M, K), 5 * M + K + ksplit)
+    ra = torch.arange(M, dtype=torch.float32) % 3 - 1
+    want = ((2 + ra.double())[:, None] * X.double() + Ad @ X.double()).float().bfloat16()
+    Xo, XoT = gpu_util.gemm_axpby(lib, A.to(DEV), X.to(DEV), 2.0, row_alpha=ra.to(DEV))
+    assert torch.equal(Xo.cpu(), want)
+    assert torch.equal(XoT.cpu(), want.T)
+    Xh = _ints((M, K), 7 * M + K, dtype=torch.float16)
+    assert torch.equal(matmul_transpose(Xh.to(DEV)).cpu(), (Xh.double() @ Xh.double().T).half())
+
+
+@pytest.mark.parametrize("M,K", [(768, 3072), (1024, 8192)])
+def test_few_tiles_long_k_chosen_by_shape(lib, knobs, M, K):
+    """Left to the library these shapes are cut along k; against the same tiles whole (KSPLIT = 1),
+    to within the rounding of the fp32 sums' different grouping, and against the fp32 product."""
+    g = torch.Generator().manual_seed(M + K)
+    X = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    auto = matmul_transpose(X)
+    knobs("FLASHMUON_KSPLIT", 1)
+    whole = matmul_transpose(X)
+    ref = X.float() @ X.float().T
+    assert torch.equal(auto, auto.T)
+    for Y in (auto, whole):
+        assert float((Y.float() - ref).norm() / ref.norm()) < 3e-3
+    assert float((auto.float() - whole.float()).norm() / ref.norm()) < 3e-3
