@@ -77,7 +77,8 @@ FM_API int fm_set_knob(int knob, long long value);
  * fm_syrk_bf16, fm_syrk_f16, fm_syrk_f32 and fm_syrk_poly_bf16, (M, K) for fm_gemm_axpby_bf16.  It holds the
  * fp32 partial tiles of output tiles whose k range is split over several workgroups: 256 KiB per
  * part, at most 256 parts (64 MiB) when the output has more 256x256 tiles than the GPU has CUs,
- * at most 768 (192 MiB) below that, and 0 for shapes that never take that schedule.
+ * at most 768 (192 MiB) below that; 16 MiB (256 parts of 64 KiB) for outputs of at most 128 tiles
+ * of 128x128 that are not whole 256x256 tiles, and 0 for shapes that never take such a schedule.
  * The calls also run with ws == NULL (or a smaller ws) on a slower schedule that needs none.
  */
 FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
