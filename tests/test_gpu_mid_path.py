@@ -138,3 +138,20 @@ def test_few_tiles_long_k_chosen_by_shape(lib, knobs, M, K):
     for Y in (auto, whole):
         assert float((Y.float() - ref).norm() / ref.norm()) < 3e-3
     assert float((auto.float() - whole.float()).norm() / ref.norm()) < 3e-3
+
+
+def test_batched_newtonschulz_with_tiles_cut_along_k(lib, knobs, no_256_path):
+    """Three matrices per launch, every 128x128 tile of every product cut into 2 parts along k: the
+    tile list and the parts' slots run over the whole batch (at most 90 x 2 parts, which the 256
+    slots of the workspace hold; with more the tiles would stay whole).  Against one matrix at a time
+    with the same cut (bitwise) and the tiles whole (to the rounding of the regrouped fp32 sums)."""
+    from flash_muon_amd import fast_newtonschulz
+    g = torch.Generator().manual_seed(21)
+    G = torch.randn(3, 384, 1280, generator=g).bfloat16().to(DEV)
+    knobs("FLASHMUON_KSPLIT", 2)
+    cut = fast_newtonschulz(G, steps=5)
+    for i in range(3):
+        assert torch.equal(cut[i], fast_newtonschulz(G[i], steps=5))
+    knobs("FLASHMUON_KSPLIT", 1)
+    whole = fast_newtonschulz(G, steps=5)
+    assert float((cut.float() - whole.float()).norm() / whole.float().norm()) < 2e-2
