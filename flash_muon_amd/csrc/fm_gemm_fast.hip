@@ -33,7 +33,7 @@ constexpr int kMaxKsplit = 16;              // base parts per tile
 // s_waitcnt vmcnt + s_barrier before the data is read.
 __device__ __forceinline__ void dma16(uint32_t voff, const void* sbase, uint32_t lds_base) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(voff), "s"(sbase), "s"(lds_base) : "memory");
+               :: "v"(voff), "s"(sbase), "s"(lds_base) : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
@@ -77,7 +77,7 @@ __device__ __forceinline__ bf16x8_t read_b(const unsigned char* smem, const Frag
 // 4 GiB too low.)
 __device__ __forceinline__ void dma16o(uint32_t voff, const void* sbase, uint32_t lds_base, int off) {
   asm volatile("s_add_i32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory", "scc");
+               :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory", "scc", "m0");
 }
 
 // The 4 NI MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The NI + 4 fragment reads of

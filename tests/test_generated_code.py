@@ -82,6 +82,18 @@ def test_every_assembly_statement_that_writes_scc_says_so():
     assert not bad, bad
 
 
+def test_every_assembly_statement_that_writes_m0_says_so():
+    """The copies set M0 themselves; declared, the register is the compiler's to avoid around them."""
+    text = open(SRC).read()
+    bad = []
+    for m in re.finditer(r"asm volatile\((.*?)\);", text, re.S):
+        body = m.group(1)
+        code = body.split("::")[0] if "::" in body else body
+        if re.search(r"\bs_[a-z0-9_]+\s+m0\b", code) and '"m0"' not in body:
+            bad.append(body.strip().split("\n")[0][:100])
+    assert not bad, bad
+
+
 def test_gemm_kernels_do_not_spill(assembly):
     """One wave per SIMD owns all 512 registers of a lane; a spill means scratch traffic inside the
     MFMA loop or the write-out."""
