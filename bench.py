@@ -168,6 +168,14 @@ def _extras(Xd, steps, warmup, torch):
         ex["torch_xxt_%d_steady_ms" % dim] = ref_s
         ex["xxt_%d_steady_speedup_vs_torch" % dim] = ref_s / ours_s
         del Xs
+    # a wide input with few output tiles and a long k (cut along k on the 128x128 path), steady state
+    Xw = synthetic.gaussian_bf16(1024, 8192, 1024).cuda()
+    ours_w = _time_gpu(lambda: matmul_transpose(Xw), 200, 100, torch)
+    ref_w = _time_gpu(lambda: torch.matmul(Xw, Xw.T), 200, 100, torch)
+    ex["xxt_1024x8192_steady_ms"] = ours_w
+    ex["torch_xxt_1024x8192_steady_ms"] = ref_w
+    ex["xxt_1024x8192_steady_speedup_vs_torch"] = ref_w / ours_w
+    del Xw
     # fast_newtonschulz(5) on the gradient-like inputs of the rectangular and the square case
     # (noise of std 1e-3 plus a rank-r spike, Frobenius-normalised; generated on the CPU from the
     # seed so that the CPU oracle sees the same bits)
