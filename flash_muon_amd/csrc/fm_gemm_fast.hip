@@ -1396,10 +1396,11 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb, MidSplit 
   for (int s = 0; s < nk; ++s) {
     wait_vmcnt<8 * (MID_STAGES - 2)>();   // my copies of stage s have landed ...
     __syncthreads();                      // ... and everybody's; stage s-1 is read out everywhere
-    {
-      const int nx = s + MID_STAGES - 1;
-      issue(nx < nk ? nx : nk - 1, nx & (MID_STAGES - 1));
-    }
+    // the 8 copies of the stage three ahead go out two per substep, an even stream of requests
+    // instead of a burst behind the barrier
+    const int nx = s + MID_STAGES - 1;
+    const int nstage = nx < nk ? nx : nk - 1;
+    const uint32_t nbase = ring + (nx & (MID_STAGES - 1)) * MID_STAGE;
     const unsigned char* sa = smem + (s & (MID_STAGES - 1)) * MID_STAGE;
     const unsigned char* sb = sa + MID_OPER;
     // the 4 fragment reads of substep ks+1 ride on the 4 MFMAs of substep ks
@@ -1424,6 +1425,13 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_kernel(GemmArgs gb, MidSplit 
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = mfma_32x32x16<F16>(fa[cur][i], fb[cur][j], acc[i][j]);
+      if (ks < 2) {
+#pragma unroll
+        for (int q = 2 * ks; q < 2 * ks + 2; ++q) dma16(voA[q], gA + nstage * BKF, nbase + q * 4096);
+      } else {
+#pragma unroll
+        for (int q = 2 * ks - 4; q < 2 * ks - 2; ++q) dma16(voB[q], gB + nstage * BKF, nbase + MID_OPER + q * 4096);
+      }
       if (ks < 3) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
