@@ -1577,26 +1577,39 @@ static bool tiled_dma_eligible(const GemmArgs& a, int tile) {
   return true;
 }
 
-// Parts per 128x128 tile along k: as many as fill the chip, of at least 4 stages each, when the
-// stages saved outweigh the fp32 round trip and the second launch (estimates in microseconds: 0.55
-// per stage, 6 for a tile's start and write-out, 10 more for the detour).
+// Parts per 128x128 tile along k, by estimate in microseconds (measured: 0.36 per stage, 4.5 for a
+// tile's start and write-out; cut, 11 for the fp32 round trip and the second launch and 0.035 per
+// part for their traffic).  At most as many parts as fill the chip, of at least 8 stages each; the
+// tiles stay whole unless the cut saves a tenth.
+static double estimate_mid_cut(long long tiles, int nk, int s) {
+  return (double)((nk + s - 1) / s) * 0.36 + 11.0 + 0.035 * (double)(tiles * s);
+}
 static int mid_ksplit(long long tiles, int nk, int grid) {
   const long long k = knob(kKnobKsplit);
-  int s = 1;
   if (k >= 1) {
-    s = (int)(k > kMaxParts ? kMaxParts : k);
-  } else if (tiles * 2 <= grid && nk >= 16) {
-    s = (int)(grid / tiles);
-    if (s > nk / 4) s = nk / 4;
-    if (s > 16) s = 16;
-    if (s < 2 || nk * 0.55 + 6.0 <= (nk / s) * 0.55 + 16.0) s = 1;
+    const int s = (int)(k > kMaxParts ? kMaxParts : k);
+    return s > nk ? nk : s;
   }
-  return s > nk ? nk : s;
+  if (tiles * 2 > grid || nk < 16) return 1;
+  int smax = (int)(grid / tiles);
+  if (smax > nk / 8) smax = nk / 8;
+  if (smax > 16) smax = 16;
+  int best = 1;
+  double t_best = 0.9 * (nk * 0.36 + 4.5);
+  for (int s = 2; s <= smax; ++s) {
+    const double t = estimate_mid_cut(tiles, nk, s);
+    if (t < t_best) { t_best = t; best = s; }
+  }
+  return best;
 }
-static double estimate_mid(long long tiles, int nk, int grid) {
+// (a stage costs 0.36 us while about half the CUs work and 0.52 when all do; a write-out with an
+// operand E costs 5 more)
+static double estimate_mid(long long tiles, int nk, int grid, bool with_e) {
   const int s = mid_ksplit(tiles, nk, grid);
-  if (s > 1) return (nk / s) * 0.55 + 16.0;
-  return (double)((tiles + grid - 1) / grid) * (nk * 0.55 + 6.0);
+  if (s > 1) return estimate_mid_cut(tiles, nk, s) + (with_e ? 5.0 : 0.0);
+  const double occ = tiles >= grid ? 1.0 : (double)tiles / grid;
+  const double stage = 0.36 + 0.36 * (occ > 0.55 ? occ - 0.55 : 0.0);
+  return (double)((tiles + grid - 1) / grid) * (nk * stage + (with_e ? 11.0 : 6.0));
 }
 
 // Estimates in microseconds, from measured costs of a k stage and of a tile's start and write-out.
@@ -1646,7 +1659,7 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   const int ksplit = auto_ksplit(tiles, nk, cus);
   const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
   const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
-  const double t_small = estimate_mid(small_tiles, nk, cus);
+  const double t_small = estimate_mid(small_tiles, nk, cus, a.E != nullptr);
   const long long half_items = (a.symmetric ? tm * tm : 2 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
   // (the 128x128 tiles keep the benefit of the doubt against half tiles)
   if (half_schedule_chosen(half_items, tiles, nk, cus) && estimate_half_round(half_items, nk, cus) < 0.9 * t_small) return true;
