@@ -31,11 +31,27 @@ inline void* usable_ws(void* ws) { return (reinterpret_cast<uintptr_t>(ws) % 256
 struct NsLayout {
   size_t sumsq, partials, pdiag, x[2], xt[2], a, p, gemm, total;
   size_t pdiag_stride;   // floats between the fp32 diagonals of consecutive matrices
+  int M, K;              // the sizes the iteration runs on: those of the matrix, or padded (below)
+  bool padded;
 };
+// A matrix whose sides are not whole 128-tiles would take the general GEMM path in every stage
+// (0.5-0.8 times the vendor GEMMs).  Its iterates live in the workspace anyway, so they are kept
+// zero-padded to whole tiles instead: zero rows and columns stay zero through every step, and the
+// tiled paths run.  Sides from 3072 on go to a multiple of 256 when that adds at most 128 (the
+// 256x256 path).
+static int ns_pad(int n) {
+  int p = (n + 127) / 128 * 128;
+  if (p >= 3072 && p % 256 != 0) p += 128;
+  return p;
+}
 NsLayout ns_layout(int batch, int rows, int cols) {
-  const size_t M = (size_t)(rows < cols ? rows : cols), K = (size_t)(rows < cols ? cols : rows);
+  const int m = rows < cols ? rows : cols, k = rows < cols ? cols : rows;
   const size_t B = (size_t)batch;
   NsLayout l;
+  l.padded = m % 128 != 0 || k % 128 != 0;
+  l.M = l.padded ? ns_pad(m) : m;
+  l.K = l.padded ? ns_pad(k) : k;
+  const size_t M = (size_t)l.M, K = (size_t)l.K;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };
   l.sumsq = take(B * 64 * sizeof(float));                 // one float per matrix, 256 bytes apart
@@ -46,7 +62,7 @@ NsLayout ns_layout(int batch, int rows, int cols) {
   l.a = take(B * M * M * 2);
   l.p = take(B * M * M * 2);
   // partial tiles of the three products of a step: two M x M (symmetric) and one M x K, `batch` each
-  const size_t g1 = gemm_fast_workspace_bytes((int)M, (int)M, batch), g2 = gemm_fast_workspace_bytes((int)M, (int)K, batch);
+  const size_t g1 = gemm_fast_workspace_bytes(l.M, l.M, batch), g2 = gemm_fast_workspace_bytes(l.M, l.K, batch);
   l.gemm = take(g1 > g2 ? g1 : g2);
   l.total = off;
   return l;
@@ -296,7 +312,8 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
   const size_t gws_bytes = l.total - l.gemm;
   hipStream_t hs = static_cast<hipStream_t>(stream);
   const bool tall = rows > cols;
-  const int M = tall ? cols : rows, K = tall ? rows : cols;
+  const bool padded = l.padded && steps > 0;
+  const int M = padded ? l.M : (tall ? cols : rows), K = padded ? l.K : (tall ? rows : cols);
   const int64_t mk = (int64_t)M * K, mm = (int64_t)M * M;
 
   // The iteration runs on X (M x K) with M <= K.  G is X when it is wide and X^T when it is
@@ -309,6 +326,8 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
     float* partials = reinterpret_cast<float*>(w + l.partials);
     for (int i = 0; i < batch; ++i)
       if (misaligned(G[i], dtype_size(dtype))) return FM_ERR_ALIGN;
+    // the padding of X and X^T (the two buffers lie next to each other)
+    if (padded && launch_fill_zero(w + l.x[0], (l.xt[0] - l.x[0]) + (size_t)batch * mk * 2, hs)) return FM_ERR_LAUNCH;
     if (launch_sumsq_batched(G, batch, dtype, rows, cols, ldg, sumsq, 64, partials, hs)) return FM_ERR_LAUNCH;
     bf16_t* d[kMaxBatch];
     bf16_t* t[kMaxBatch];
@@ -357,6 +376,9 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
     if (!last) {
       g.C = Xn; g.c_rs = K; g.bs_c = mk;
       g.C2 = XTn; g.c2_rs = M; g.bs_c2 = mk;
+    } else if (padded) {  // the orientation the caller wants, into the workspace, and from there out
+      if (!tall) { g.C = Xn; g.c_rs = K; g.bs_c = mk; }
+      else { g.C2 = XTn; g.c2_rs = M; g.bs_c2 = mk; }
     } else if (!tall) {   // the result has G's shape: X itself
       g.C = static_cast<bf16_t*>(out[0]); g.c_rs = ldout; g.use_c_list = 1;
       for (int i = 0; i < batch; ++i) g.c_list[i] = static_cast<bf16_t*>(out[i]);
@@ -366,6 +388,11 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
     }
     if (launch_gemm_nt(g, gws, gws_bytes, hs)) return FM_ERR_LAUNCH;
     X = Xn; XT = XTn;
+  }
+  if (padded) {
+    bf16_t* o[kMaxBatch];
+    for (int i = 0; i < batch; ++i) o[i] = static_cast<bf16_t*>(out[i]);
+    if (launch_copy2d_batched(tall ? XT : X, tall ? M : K, mk, o, ldout, batch, rows, cols, hs)) return FM_ERR_LAUNCH;
   }
   return FM_OK;
 }

@@ -366,4 +366,52 @@ int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float
   return launch_weight_update_batched(&p, &u, 1, p_dtype, n, decay_mul, alpha, stream);
 }
 
+// ---- zero fill and 2-D copy, for the padded copies Newton-Schulz keeps of ragged matrices --------
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint4* p, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) p[i] = uint4{0u, 0u, 0u, 0u};
+}
+
+int launch_fill_zero(void* p, size_t bytes, hipStream_t stream) {   // p 16-byte aligned, bytes a multiple of 16
+  const int64_t n16 = (int64_t)(bytes / 16);
+  if (n16 == 0) return 0;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_grid(n16)), dim3(256), 0, stream, static_cast<uint4*>(p), n16);
+  return (int)hipGetLastError();
+}
+
+// dst[b][r][c] = src[b * bs_src + r * lds + c] for r < rows, c < cols (16-bit elements);
+// blockIdx.y strides over the rows, blockIdx.z is the matrix; `vec`: 8 elements per lane
+// (everything 16-byte aligned)
+__global__ __launch_bounds__(256) void copy2d_kernel(const unsigned short* src, int64_t lds, int64_t bs_src,
+                                                     PtrList dl, int64_t ldd, int rows, int cols, int vec) {
+  const int t = (int)blockIdx.x * 256 + (int)threadIdx.x;
+  for (int r = (int)blockIdx.y; r < rows; r += (int)gridDim.y) {
+    const unsigned short* s = src + (int64_t)blockIdx.z * bs_src + (int64_t)r * lds;
+    unsigned short* d = reinterpret_cast<unsigned short*>(dl.p[blockIdx.z]) + (int64_t)r * ldd;
+    if (vec) {
+      if (t * 8 < cols) reinterpret_cast<uint4*>(d)[t] = reinterpret_cast<const uint4*>(s)[t];
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int c = t + e * (int)gridDim.x * 256;
+        if (c < cols) d[c] = s[c];
+      }
+    }
+  }
+}
+
+int launch_copy2d_batched(const bf16_t* src, int64_t lds, int64_t bs_src, bf16_t* const* dst, int64_t ldd,
+                          int batch, int rows, int cols, hipStream_t stream) {
+  int vec = cols % 8 == 0 && ldd % 8 == 0 && lds % 8 == 0 && bs_src % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+  PtrList dl = {};
+  for (int i = 0; i < batch; ++i) {
+    dl.p[i] = dst[i];
+    vec = vec && (reinterpret_cast<uintptr_t>(dst[i]) & 15) == 0;
+  }
+  dim3 grid((unsigned)((cols + 2047) / 2048), (unsigned)(rows < 65535 ? rows : 65535), (unsigned)batch);
+  hipLaunchKernelGGL(copy2d_kernel, grid, dim3(256), 0, stream, reinterpret_cast<const unsigned short*>(src), lds, bs_src,
+                     dl, ldd, rows, cols, vec);
+  return (int)hipGetLastError();
+}
+
 }  // namespace fm

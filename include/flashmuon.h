@@ -182,7 +182,9 @@ FM_API int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int6
  * (row stride ldg), out is rows x cols bf16 (row stride ldout).  Runs fm_sumsq,
  * fm_scale_cast_bf16 and `steps` x (fm_syrk_bf16, fm_syrk_poly_bf16, fm_gemm_axpby_bf16) on
  * `stream`, iterating on the wide orientation (M = min(rows, cols)).  steps == 0 returns the
- * normalised input.  out must not overlap G.
+ * normalised input.  out must not overlap G.  A matrix whose sides are not whole multiples of 128
+ * is iterated on zero-padded to whole tiles inside the workspace (zero rows and columns stay zero
+ * through every step) and the rows x cols part is copied out at the end.
  * Replaces fast_newtonschulz: flash_muon/muon.py:6-33.
  */
 FM_API size_t fm_newtonschulz_workspace_bytes(int rows, int cols);
