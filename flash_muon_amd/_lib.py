@@ -29,6 +29,7 @@ SIGNATURES = {
     "fm_version": (ctypes.c_char_p, []),
     "fm_set_knob": (_i32, [_i32, ctypes.c_longlong]),
     "fm_gemm_workspace_bytes": (_sz, [_i32, _i32]),
+    "fm_syrk_workspace_bytes": (_sz, [_i32, _i32]),
     "fm_syrk_bf16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),
     "fm_syrk_bf16_static": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp]),
     "fm_syrk_f16": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _sz, _vp]),

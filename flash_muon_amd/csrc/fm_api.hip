@@ -120,8 +120,33 @@ size_t fm_gemm_workspace_bytes(int rows_out, int cols_out) {
 
 int fm_set_knob(int which, long long value) { return set_knob(which, value) == 0 ? FM_OK : FM_ERR_SHAPE; }
 
+// X * X^T of a matrix whose sides are not whole 128-tiles, through zero-padded copies: X padded in
+// the workspace, the product of that on the tiled paths into a padded Y beside it, and the M x M
+// part copied out.  Pays from about a million elements of X on (below that the general path's single
+// launch wins); 16-bit elements only.
+struct SyrkPad { int Mp, Kp; size_t x, y, gemm, total; };
+constexpr int64_t kSyrkPadMinElems = 256 * 256;
+static bool syrk_pad_layout(int M, int K, SyrkPad* p) {
+  if (M <= 0 || K <= 0 || (M % 128 == 0 && K % 128 == 0) || (int64_t)M * K < kSyrkPadMinElems) return false;
+  p->Mp = ns_pad(M);
+  p->Kp = (K + 127) / 128 * 128;
+  p->x = 0;
+  p->y = align_up((size_t)p->Mp * p->Kp * 2, 256);
+  p->gemm = p->y + align_up((size_t)p->Mp * p->Mp * 2, 256);
+  p->total = p->gemm + gemm_fast_workspace_bytes(p->Mp, p->Mp, 1);
+  return true;
+}
+
+size_t fm_syrk_workspace_bytes(int M, int K) {
+  if (M <= 0) return 0;
+  const size_t plain = gemm_fast_workspace_bytes(M, M, 1);
+  SyrkPad p;
+  if (!syrk_pad_layout(M, K, &p)) return plain;
+  return p.total > plain ? p.total : plain;
+}
+
 static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
-                     void* ws, size_t ws_bytes, fm_stream_t stream, int elem) {
+                     void* ws, size_t ws_bytes, fm_stream_t stream, int elem, bool may_pad = true) {
   if (M < 0 || K < 0) return FM_ERR_SHAPE;
   if (M == 0) return FM_OK;
   if (!X && K > 0) return FM_ERR_NULL;
@@ -145,14 +170,33 @@ static int syrk_impl(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64
     y.hi = y.lo + (uintptr_t)(((M - 1) * (ar + ac) + 1) * es);
     if (K > 0 && overlaps(mat_range(X, M, K, ldx, es), y)) return FM_ERR_ALIAS;
   }
+  hipStream_t hs = static_cast<hipStream_t>(stream);
   GemmArgs a = {};
-  a.A = a.B = static_cast<const bf16_t*>(X); a.lda = a.ldb = ldx;
   a.E = nullptr; a.lde = 0;
+  a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1; a.elem = elem;
+  SyrkPad p;
+  // Y is symmetric, so a unit stride in either direction makes its lines rows for the copy out
+  const int64_t ldy = ldy_col == 1 ? ldy_row : ldy_row == 1 ? ldy_col : 0;
+  if (may_pad && elem != kElemF32 && ldy >= M && usable_ws(ws) && syrk_pad_layout(M, K, &p) && ws_bytes >= p.total &&
+      !overlaps(mat_range(X, M, K, ldx, es), Range{reinterpret_cast<uintptr_t>(ws), reinterpret_cast<uintptr_t>(ws) + p.total}) &&
+      !overlaps(mat_range(Y, M, M, ldy, es), Range{reinterpret_cast<uintptr_t>(ws), reinterpret_cast<uintptr_t>(ws) + p.total})) {
+    unsigned char* w = static_cast<unsigned char*>(ws);
+    bf16_t* Xp = reinterpret_cast<bf16_t*>(w + p.x);
+    bf16_t* Yp = reinterpret_cast<bf16_t*>(w + p.y);
+    bf16_t* xl[1] = {Xp};
+    bf16_t* yl[1] = {static_cast<bf16_t*>(Y)};
+    if (launch_copy2d_batched(static_cast<const bf16_t*>(X), ldx, 0, xl, p.Kp, 1, M, K, p.Mp, p.Kp, hs)) return FM_ERR_LAUNCH;
+    a.A = a.B = Xp; a.lda = a.ldb = p.Kp;
+    a.C = a.C2 = Yp; a.c_rs = a.c2_rs = p.Mp; a.c_cs = a.c2_cs = 1;
+    a.Ma = a.Nb = p.Mp; a.Kc = p.Kp;
+    if (launch_gemm_nt(a, w + p.gemm, ws_bytes - p.gemm, hs)) return FM_ERR_LAUNCH;
+    return hip_status(launch_copy2d_batched(Yp, p.Mp, 0, yl, ldy, 1, M, M, M, M, hs));
+  }
+  a.A = a.B = static_cast<const bf16_t*>(X); a.lda = a.ldb = ldx;
   a.C = a.C2 = static_cast<bf16_t*>(Y);
   a.c_rs = a.c2_rs = ldy_row; a.c_cs = a.c2_cs = ldy_col;
   a.Ma = a.Nb = M; a.Kc = K;
-  a.alpha = 0.0f; a.beta = 1.0f; a.symmetric = 1; a.elem = elem;
-  return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, static_cast<hipStream_t>(stream)));
+  return hip_status(launch_gemm_nt(a, usable_ws(ws), ws_bytes, hs));
 }
 
 int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
@@ -166,7 +210,8 @@ int fm_syrk_bf16_static(const void* X, int64_t ldx, void* Y, int64_t ldy_row, in
   void* scratch = nullptr;
   const int rc = static_scratch(&scratch);
   if (rc != FM_OK) return rc;
-  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, scratch, kStaticScratchBytes, stream, kElemBf16);
+  // always the schedules of fm_syrk_bf16 with a workspace of fm_gemm_workspace_bytes(M, M), bit for bit
+  return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, scratch, kStaticScratchBytes, stream, kElemBf16, false);
 }
 
 int fm_syrk_f16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col, int M, int K,
@@ -392,7 +437,8 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
   if (padded) {
     bf16_t* o[kMaxBatch];
     for (int i = 0; i < batch; ++i) o[i] = static_cast<bf16_t*>(out[i]);
-    if (launch_copy2d_batched(tall ? XT : X, tall ? M : K, mk, o, ldout, batch, rows, cols, hs)) return FM_ERR_LAUNCH;
+    if (launch_copy2d_batched(tall ? XT : X, tall ? M : K, mk, o, ldout, batch, rows, cols, rows, cols, hs))
+      return FM_ERR_LAUNCH;
   }
   return FM_OK;
 }

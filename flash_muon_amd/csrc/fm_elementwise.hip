@@ -379,38 +379,52 @@ int launch_fill_zero(void* p, size_t bytes, hipStream_t stream) {   // p 16-byte
   return (int)hipGetLastError();
 }
 
-// dst[b][r][c] = src[b * bs_src + r * lds + c] for r < rows, c < cols (16-bit elements);
-// blockIdx.y strides over the rows, blockIdx.z is the matrix; `vec`: 8 elements per lane
-// (everything 16-byte aligned)
+// dst[b] (rows_d x cols_d, pitch ldd) = src[b] (rows x cols at src + b * bs_src, pitch lds) where
+// that exists and zero elsewhere, 16-bit elements.  A lane moves 8 consecutive elements of a row, as
+// one 16-byte access on a side that is aligned for it (`src_vec`, `dst_vec`) and element by element
+// otherwise; blockIdx.y strides over the rows, blockIdx.z is the matrix.
 __global__ __launch_bounds__(256) void copy2d_kernel(const unsigned short* src, int64_t lds, int64_t bs_src,
-                                                     PtrList dl, int64_t ldd, int rows, int cols, int vec) {
-  const int t = (int)blockIdx.x * 256 + (int)threadIdx.x;
-  for (int r = (int)blockIdx.y; r < rows; r += (int)gridDim.y) {
-    const unsigned short* s = src + (int64_t)blockIdx.z * bs_src + (int64_t)r * lds;
-    unsigned short* d = reinterpret_cast<unsigned short*>(dl.p[blockIdx.z]) + (int64_t)r * ldd;
-    if (vec) {
-      if (t * 8 < cols) reinterpret_cast<uint4*>(d)[t] = reinterpret_cast<const uint4*>(s)[t];
+                                                     PtrList dl, int64_t ldd, int rows, int cols, int rows_d,
+                                                     int cols_d, int src_vec, int dst_vec) {
+  const int c0 = ((int)blockIdx.x * 256 + (int)threadIdx.x) * 8;
+  if (c0 >= cols_d) return;
+  for (int r = (int)blockIdx.y; r < rows_d; r += (int)gridDim.y) {
+    union { uint4 v; unsigned short e[8]; } u;
+    u.v = uint4{0u, 0u, 0u, 0u};
+    if (r < rows) {
+      const unsigned short* s = src + (int64_t)blockIdx.z * bs_src + (int64_t)r * lds + c0;
+      if (src_vec && c0 + 8 <= cols) {
+        u.v = *reinterpret_cast<const uint4*>(s);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (c0 + e < cols) u.e[e] = s[e];
+      }
+    }
+    unsigned short* d = reinterpret_cast<unsigned short*>(dl.p[blockIdx.z]) + (int64_t)r * ldd + c0;
+    if (dst_vec && c0 + 8 <= cols_d) {
+      *reinterpret_cast<uint4*>(d) = u.v;
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int c = t + e * (int)gridDim.x * 256;
-        if (c < cols) d[c] = s[c];
-      }
+      for (int e = 0; e < 8; ++e)
+        if (c0 + e < cols_d) d[e] = u.e[e];
     }
   }
 }
 
 int launch_copy2d_batched(const bf16_t* src, int64_t lds, int64_t bs_src, bf16_t* const* dst, int64_t ldd,
-                          int batch, int rows, int cols, hipStream_t stream) {
-  int vec = cols % 8 == 0 && ldd % 8 == 0 && lds % 8 == 0 && bs_src % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+                          int batch, int rows, int cols, int rows_d, int cols_d, hipStream_t stream) {
+  if (batch <= 0 || rows_d <= 0 || cols_d <= 0) return 0;
+  const int src_vec = lds % 8 == 0 && bs_src % 8 == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0;
+  int dst_vec = ldd % 8 == 0;
   PtrList dl = {};
   for (int i = 0; i < batch; ++i) {
     dl.p[i] = dst[i];
-    vec = vec && (reinterpret_cast<uintptr_t>(dst[i]) & 15) == 0;
+    dst_vec = dst_vec && (reinterpret_cast<uintptr_t>(dst[i]) & 15) == 0;
   }
-  dim3 grid((unsigned)((cols + 2047) / 2048), (unsigned)(rows < 65535 ? rows : 65535), (unsigned)batch);
+  dim3 grid((unsigned)((cols_d + 2047) / 2048), (unsigned)(rows_d < 65535 ? rows_d : 65535), (unsigned)batch);
   hipLaunchKernelGGL(copy2d_kernel, grid, dim3(256), 0, stream, reinterpret_cast<const unsigned short*>(src), lds, bs_src,
-                     dl, ldd, rows, cols, vec);
+                     dl, ldd, rows, cols, rows_d, cols_d, src_vec, dst_vec);
   return (int)hipGetLastError();
 }
 

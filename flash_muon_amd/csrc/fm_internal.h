@@ -149,7 +149,7 @@ int launch_weight_update_batched(void* const* p, const bf16_t* const* u, int bat
                                  float decay_mul, float alpha, hipStream_t stream);
 int launch_fill_zero(void* p, size_t bytes, hipStream_t stream);
 int launch_copy2d_batched(const bf16_t* src, int64_t lds, int64_t bs_src, bf16_t* const* dst, int64_t ldd,
-                          int batch, int rows, int cols, hipStream_t stream);
+                          int batch, int rows, int cols, int rows_d, int cols_d, hipStream_t stream);
 int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,
                              int nesterov, hipStream_t stream);
 int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float decay_mul,

@@ -46,7 +46,7 @@ def matmul_transpose_assign(d_in, d_out):
     if M > 1 and (min(rs, cs) == 0 or max(rs, cs) < M * min(rs, cs)):
         dst = torch.empty((M, M), device=d_in.device, dtype=d_in.dtype)
     with torch.cuda.device(d_in.device):
-        need = 0 if d_in.dtype == torch.float32 else lib.fm_gemm_workspace_bytes(M, M)
+        need = 0 if d_in.dtype == torch.float32 else lib.fm_syrk_workspace_bytes(M, K)
         ws, ws_bytes = _lib.gemm_workspace(need, d_in.device)
         st = getattr(lib, entry)(d_in.data_ptr(), ldx, dst.data_ptr(),
                                  dst.stride(0) if M > 1 else M, dst.stride(1) if M > 1 else 1,

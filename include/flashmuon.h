@@ -95,6 +95,15 @@ FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
 FM_API int fm_syrk_bf16(const void* X, int64_t ldx, void* Y, int64_t ldy_row, int64_t ldy_col,
                  int M, int K, void* ws, size_t ws_bytes, fm_stream_t stream);
 
+/* Scratch for fm_syrk_bf16 and fm_syrk_f16 by the shape of X: fm_gemm_workspace_bytes(M, M), and for
+ * an X whose sides are not whole multiples of 128 also room for a zero-padded copy of X and the padded
+ * product, so that such shapes run on the tiled schedules too (copied in, multiplied, the M x M part
+ * copied out: three launches) instead of the general one.  With less than this the calls still run,
+ * on the schedule that the scratch they get allows.  No counterpart in the reference, whose masked
+ * loads and stores take any shape (flash_muon/matmul_transpose_triton.py:48-52, 70-75).
+ */
+FM_API size_t fm_syrk_workspace_bytes(int M, int K);
+
 /* fm_syrk_bf16 for callers that cannot allocate or hand over scratch memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments and results as fm_syrk_bf16 minus ws / ws_bytes: the partial tiles go
