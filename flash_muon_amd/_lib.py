@@ -108,7 +108,8 @@ _gemm_ws = {}
 
 
 def gemm_workspace(nbytes, device):
-    """The partial-tile scratch of the single GEMM-shaped calls (at most 192 MiB), kept per device
+    """The scratch of the single GEMM-shaped calls (partial tiles, at most 192 MiB; for a product
+    whose sides are not whole tiles also its zero-padded operand and result), kept per device
     and stream: calls on one stream are ordered, so they can share it, and nothing is allocated
     per call."""
     if nbytes == 0:

@@ -10,10 +10,12 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def test_graph_replays_match_eager():
-    G = synthetic.gradient_like_bf16(512, 1536, 8, 41).to(DEV)
-    X = synthetic.gaussian_bf16(768, 1024, 42).to(DEV)
-    Y = torch.empty(768, 768, dtype=torch.bfloat16, device=DEV)
+# whole tiles, and sides that are not (zero-padded copies in the workspace: a fill kernel and copies)
+@pytest.mark.parametrize("gshape,xshape", [((512, 1536), (768, 1024)), ((500, 1500), (700, 1000))])
+def test_graph_replays_match_eager(gshape, xshape):
+    G = synthetic.gradient_like_bf16(gshape[0], gshape[1], 8, 41).to(DEV)
+    X = synthetic.gaussian_bf16(xshape[0], xshape[1], 42).to(DEV)
+    Y = torch.empty(xshape[0], xshape[0], dtype=torch.bfloat16, device=DEV)
     want_ns = fast_newtonschulz(G, 5)
     want_y = torch.empty_like(Y)
     matmul_transpose_assign(X, want_y)
@@ -41,7 +43,7 @@ def test_graph_replays_match_eager():
         assert torch.equal(fast_newtonschulz(G, 5), want_ns)
         torch.cuda.synchronize()
     # new input values in place: the graph reads the same buffers
-    G2 = synthetic.gradient_like_bf16(512, 1536, 8, 43).to(DEV)
+    G2 = synthetic.gradient_like_bf16(gshape[0], gshape[1], 8, 43).to(DEV)
     G.copy_(G2)
     graph.replay()
     torch.cuda.synchronize()
