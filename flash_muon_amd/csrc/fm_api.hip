@@ -37,20 +37,24 @@ struct NsLayout {
 // A matrix whose sides are not whole 128-tiles would take the general GEMM path in every stage
 // (0.5-0.8 times the vendor GEMMs).  Its iterates live in the workspace anyway, so they are kept
 // zero-padded to whole tiles instead: zero rows and columns stay zero through every step, and the
-// tiled paths run.  Sides from 3072 on go to a multiple of 256 when that adds at most 128 (the
-// 256x256 path).
+// tiled paths run.  From 23 tiles of 128 on the short side, whole 256x256 tiles pay for up to 128
+// more rows and columns (five steps at 3200^2 0.96 ms, at 3328^2 0.78; 5248^2 3.27, 5376^2 2.61;
+// 2688^2 and 2816^2 both 0.50), so there both sides go to multiples of 256, also when they are
+// whole multiples of 128.
+constexpr int kPad256From = 2944;
 static int ns_pad(int n) {
   int p = (n + 127) / 128 * 128;
-  if (p >= 3072 && p % 256 != 0) p += 128;
+  if (p >= kPad256From && p % 256 != 0) p += 128;
   return p;
 }
 NsLayout ns_layout(int batch, int rows, int cols) {
   const int m = rows < cols ? rows : cols, k = rows < cols ? cols : rows;
   const size_t B = (size_t)batch;
   NsLayout l;
-  l.padded = m % 128 != 0 || k % 128 != 0;
-  l.M = l.padded ? ns_pad(m) : m;
-  l.K = l.padded ? ns_pad(k) : k;
+  l.M = ns_pad(m);
+  l.K = (k + 127) / 128 * 128;
+  if (l.M >= kPad256From) l.K = (k + 255) / 256 * 256;
+  l.padded = l.M != m || l.K != k;
   const size_t M = (size_t)l.M, K = (size_t)l.K;
   size_t off = 0;
   auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes, 256); return o; };

@@ -94,12 +94,33 @@ def test_batched_matches_single_and_leaves_strided_output_alone(lib, rows, cols)
         assert oracle.rel_fro(obuf[i, :, :cols], oracle.newtonschulz(Gs[i], 5)) < TOL
 
 
-def test_large_ragged_singular_values_land_in_band():
-    # too large for the oracle in seconds: the property the iteration exists for
-    G = torch.randn(2000, 3000, device=DEV, generator=torch.Generator(DEV).manual_seed(5)).bfloat16()
-    O = fast_newtonschulz(G, 5).float()
-    s = torch.linalg.svdvals(O)
-    print("2000x3000: singular values in [%.3f, %.3f]" % (float(s.min()), float(s.max())), flush=True)
-    assert float(s.max()) < 1.25 and float(s.min()) > 0.3
-    back = fast_newtonschulz(G.T.contiguous(), 5)
-    assert torch.equal(back.T, O.bfloat16())
+def _ns_fp32_on_gpu(G, steps=5):
+    """muon.py:15-32 in fp32 with torch's GEMMs on the GPU, for sizes the CPU oracle needs minutes for."""
+    a, b, c = oracle.NS_COEFFS
+    X = G.float()
+    tall = X.size(0) > X.size(1)
+    X = X.T if tall else X
+    X = X / (X.norm() + 1e-7)
+    for _ in range(steps):
+        A = X @ X.T
+        X = a * X + (b * A + c * (A @ A)) @ X
+    return X.T if tall else X
+
+
+@pytest.mark.parametrize("rows,cols", [(2000, 3000), (3200, 3200), (2944, 4500), (4600, 3000)])
+def test_large_sides_singular_values_land_in_band(rows, cols):
+    # too large for the oracle in seconds (3200 is a whole number of 128-tiles, which the iteration
+    # pads to whole 256-tiles): the property the iteration exists for, the transposed problem bit for
+    # bit, and the fp32 iteration with torch's GEMMs on the same device within the oracle's tolerance
+    G = torch.randn(rows, cols, device=DEV, generator=torch.Generator(DEV).manual_seed(5)).bfloat16()
+    O = fast_newtonschulz(G, 5)
+    assert O.shape == G.shape
+    s = torch.linalg.svdvals(O.float())
+    print("%dx%d: singular values in [%.3f, %.3f]" % (rows, cols, float(s.min()), float(s.max())), flush=True)
+    assert float(s.max()) < 1.25
+    if rows != cols:                          # a square Gaussian matrix has singular values near zero
+        assert float(s.min()) > 0.3
+        assert torch.equal(fast_newtonschulz(G.T.contiguous(), 5).T, O)
+    err = oracle.rel_fro(O, _ns_fp32_on_gpu(G))
+    print("against fp32 on the GPU: rel_fro %.3e" % err, flush=True)
+    assert err < TOL
