@@ -92,8 +92,35 @@ def dtype_code(dtype):
         raise TypeError("unsupported dtype %s (bfloat16, float16, float32 are supported)" % dtype)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device):
+    """The hipStream_t of torch's current stream on `device`, as an integer."""
+    if _raw_stream is not None:      # the same value without building a Stream object (a few us per call)
+        idx = torch.device(device).index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def on_device(device):
+    """Context that makes `device` the current one for the kernel launches of a call; nothing to
+    enter or leave when it is current already."""
+    idx = torch.device(device).index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(idx)
 
 
 def workspace(nbytes, device):
@@ -107,14 +134,14 @@ def workspace(nbytes, device):
 _gemm_ws = {}
 
 
-def gemm_workspace(nbytes, device):
+def gemm_workspace(nbytes, device, stream=None):
     """The scratch of the single GEMM-shaped calls (partial tiles, at most 192 MiB; for a product
     whose sides are not whole tiles also its zero-padded operand and result), kept per device
     and stream: calls on one stream are ordered, so they can share it, and nothing is allocated
     per call."""
     if nbytes == 0:
         return None, 0
-    key = (torch.device(device).index, stream_ptr(device))
+    key = (torch.device(device).index, stream_ptr(device) if stream is None else stream)
     ws = _gemm_ws.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = _gemm_ws[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)

@@ -45,13 +45,13 @@ def matmul_transpose_assign(d_in, d_out):
     dst = d_out
     if M > 1 and (min(rs, cs) == 0 or max(rs, cs) < M * min(rs, cs)):
         dst = torch.empty((M, M), device=d_in.device, dtype=d_in.dtype)
-    with torch.cuda.device(d_in.device):
+    with _lib.on_device(d_in.device):
+        stream = _lib.stream_ptr(d_in.device)
         need = 0 if d_in.dtype == torch.float32 else lib.fm_syrk_workspace_bytes(M, K)
-        ws, ws_bytes = _lib.gemm_workspace(need, d_in.device)
+        ws, ws_bytes = _lib.gemm_workspace(need, d_in.device, stream)
         st = getattr(lib, entry)(d_in.data_ptr(), ldx, dst.data_ptr(),
                                  dst.stride(0) if M > 1 else M, dst.stride(1) if M > 1 else 1,
-                                 M, K, ws.data_ptr() if ws is not None else None, ws_bytes,
-                                 _lib.stream_ptr(d_in.device))
+                                 M, K, ws.data_ptr() if ws is not None else None, ws_bytes, stream)
     _lib.check(entry, st)
     if dst is not d_out:
         d_out.copy_(dst)

@@ -40,7 +40,7 @@ def _newtonschulz_into(Gs, outs, steps):
     ldo = outs[0].stride(0) if rows > 1 else cols
     g_ptrs = (ctypes.c_void_p * n)(*[g.data_ptr() for g in Gs])
     o_ptrs = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
-    with torch.cuda.device(G0.device):
+    with _lib.on_device(G0.device):
         ws, ws_bytes = _lib.workspace(lib.fm_newtonschulz_batched_workspace_bytes(n, rows, cols), G0.device)
         st = lib.fm_newtonschulz_batched_bf16(g_ptrs, _lib.dtype_code(G0.dtype), n, rows, cols, ldg,
                                               o_ptrs, ldo, steps, a, b, c, NS_EPS,
@@ -203,7 +203,7 @@ class Muon(torch.optim.Optimizer):
                         bufs.append(buf)
                     # buf.lerp_(g, 1 - mu); g.lerp_(buf, mu) in place on p.grad (muon.py:99-100),
                     # one launch for the chunk
-                    with torch.cuda.device(dev):
+                    with _lib.on_device(dev):
                         st = lib.fm_momentum_nesterov_batched(
                             (ctypes.c_void_p * n)(*[t.data_ptr() for t in gcs]),
                             (ctypes.c_void_p * n)(*[t.data_ptr() for t in bufs]),
@@ -226,7 +226,7 @@ class Muon(torch.optim.Optimizer):
                     # one launch for the chunk (same shape, so the same scale)
                     pcs = [p if p.is_contiguous() else p.contiguous() for p in chunk]
                     alpha = -lr * max(1, chunk[0].size(-2) / chunk[0].size(-1)) ** 0.5
-                    with torch.cuda.device(dev):
+                    with _lib.on_device(dev):
                         st = lib.fm_weight_update_batched(
                             (ctypes.c_void_p * n)(*[t.data_ptr() for t in pcs]), _lib.dtype_code(pcs[0].dtype),
                             (ctypes.c_void_p * n)(*[staging[i].data_ptr() for i in range(n)]),
