@@ -37,11 +37,15 @@ struct NsLayout {
 // A matrix whose sides are not whole 128-tiles would take the general GEMM path in every stage
 // (0.5-0.8 times the vendor GEMMs).  Its iterates live in the workspace anyway, so they are kept
 // zero-padded to whole tiles instead: zero rows and columns stay zero through every step, and the
-// tiled paths run.  From 23 tiles of 128 on the short side, whole 256x256 tiles pay for up to 128
-// more rows and columns (five steps at 3200^2 0.96 ms, at 3328^2 0.78; 5248^2 3.27, 5376^2 2.61;
-// 2688^2 and 2816^2 both 0.50), so there both sides go to multiples of 256, also when they are
-// whole multiples of 128.
-constexpr int kPad256From = 2944;
+// tiled paths run.  Whole 256x256 tiles pay for up to 128 more rows and columns, also where the
+// sides are whole multiples of 128 already, once the 256x256 path has enough of them: for a single
+// matrix from a short side of 2176 on (five steps at 2176^2 0.43 ms, at 2304^2 0.41; 3200^2 0.96
+// and 3328^2 0.78; 5248^2 3.27 and 5376^2 2.61; but 1920^2 0.31 and 2048^2 0.34), for a batch as
+// soon as its 256x256 tiles fill the GPU (32 of 1664^2 4.6 ms, of 1792^2 4.2; 2688 x 7168 36 and
+// 2816 x 7168 26).  The long side alone goes to a multiple of 256 where the short one is one already
+// (32 of 2048 x 5504 15.4 ms, of 2048 x 5632 11.9; one matrix 0.72 and 0.59; below 1536 rows a single
+// matrix gains nothing).
+constexpr int kPad256From = 2944;       // the stand-alone product: there the copies have to be paid for
 static int ns_pad(int n) {
   int p = (n + 127) / 128 * 128;
   if (p >= kPad256From && p % 256 != 0) p += 128;
@@ -51,9 +55,14 @@ NsLayout ns_layout(int batch, int rows, int cols) {
   const int m = rows < cols ? rows : cols, k = rows < cols ? cols : rows;
   const size_t B = (size_t)batch;
   NsLayout l;
-  l.M = ns_pad(m);
+  l.M = (m + 127) / 128 * 128;
   l.K = (k + 127) / 128 * 128;
-  if (l.M >= kPad256From) l.K = (k + 255) / 256 * 256;
+  {
+    const int64_t t = (l.M + 255) / 256;
+    const bool both = l.M >= 2176 || (l.M >= 1152 && (int64_t)batch * t * (t + 1) / 2 >= 120);
+    if (both) l.M = (int)t * 256;
+    if (l.M % 256 == 0 && (both || l.M >= 1536 || (batch >= 4 && l.M >= 768))) l.K = (k + 255) / 256 * 256;
+  }
   l.padded = l.M != m || l.K != k;
   const size_t M = (size_t)l.M, K = (size_t)l.K;
   size_t off = 0;

@@ -192,7 +192,7 @@ FM_API int fm_scale_cast_bf16(const void* G, int dtype, int rows, int cols, int6
  * fm_scale_cast_bf16 and `steps` x (fm_syrk_bf16, fm_syrk_poly_bf16, fm_gemm_axpby_bf16) on
  * `stream`, iterating on the wide orientation (M = min(rows, cols)).  steps == 0 returns the
  * normalised input.  out must not overlap G.  A matrix whose sides are not whole multiples of 128
- * (of 256 when the shorter side is 2944 or more) is iterated on zero-padded to whole tiles inside the workspace (zero rows and columns stay zero
+ * (of 256 where whole 256x256 tiles are estimated to pay for the padding) is iterated on zero-padded to whole tiles inside the workspace (zero rows and columns stay zero
  * through every step) and the rows x cols part is copied out at the end.
  * Replaces fast_newtonschulz: flash_muon/muon.py:6-33.
  */

@@ -94,6 +94,20 @@ def test_batched_matches_single_and_leaves_strided_output_alone(lib, rows, cols)
         assert oracle.rel_fro(obuf[i, :, :cols], oracle.newtonschulz(Gs[i], 5)) < TOL
 
 
+def test_batch_padded_to_256_tiles_where_a_single_matrix_is_not():
+    # eight matrices of 1280 x 1408 fill the GPU with 256x256 tiles, so the batch runs on 1280 x 1536;
+    # a single one stays on 128x128 tiles of 1280 x 1408: same results within the oracle's tolerance
+    G = torch.stack([synthetic.gradient_like_bf16(1280, 1408, 8, 60 + i) for i in range(8)]).to(DEV)
+    got = fast_newtonschulz(G, 5)
+    assert got.shape == G.shape
+    for i in (0, 7):
+        ref = oracle.newtonschulz(G[i].cpu(), 5)
+        assert oracle.rel_fro(got[i], ref) < TOL
+        assert oracle.rel_fro(fast_newtonschulz(G[i], 5), ref) < TOL
+    tall = fast_newtonschulz(G.mT.contiguous(), 5)
+    assert torch.equal(tall.mT, got)
+
+
 def _ns_fp32_on_gpu(G, steps=5):
     """muon.py:15-32 in fp32 with torch's GEMMs on the GPU, for sizes the CPU oracle needs minutes for."""
     a, b, c = oracle.NS_COEFFS
