@@ -384,8 +384,6 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
     float* partials = reinterpret_cast<float*>(w + l.partials);
     for (int i = 0; i < batch; ++i)
       if (misaligned(G[i], dtype_size(dtype))) return FM_ERR_ALIGN;
-    // the padding of X and X^T (the two buffers lie next to each other)
-    if (padded && launch_fill_zero(w + l.x[0], (l.xt[0] - l.x[0]) + (size_t)batch * mk * 2, hs)) return FM_ERR_LAUNCH;
     if (launch_sumsq_batched(G, batch, dtype, rows, cols, ldg, sumsq, 64, partials, hs)) return FM_ERR_LAUNCH;
     bf16_t* d[kMaxBatch];
     bf16_t* t[kMaxBatch];
@@ -395,8 +393,10 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
       else            { d[i] = XT + i * mk; t[i] = X + i * mk; }
     }
     const int64_t ldd = steps == 0 ? ldout : (!tall ? K : M), ldt = !tall ? M : K;
+    // with padding: G's orientation is (tall ? K x M : M x K) there, and what lies beyond G is zeroed
     if (launch_scale_cast_batched(G, batch, dtype, rows, cols, ldg, sumsq, 64, eps, d, ldd,
-                                  steps == 0 ? nullptr : t, ldt, hs))
+                                  steps == 0 ? nullptr : t, ldt, hs, padded ? (tall ? K : M) : rows,
+                                  padded ? (tall ? M : K) : cols))
       return FM_ERR_LAUNCH;
   }
   if (steps == 0) return FM_OK;

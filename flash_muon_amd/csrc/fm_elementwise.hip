@@ -129,9 +129,11 @@ int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, floa
 
 // ---- normalise, cast, transpose -----------------------------------------------------------------
 // One 64x64 tile of G per block: D gets the tile in place, T gets it transposed through LDS.
+// D is rows_p x cols_p and T cols_p x rows_p with rows_p >= rows, cols_p >= cols: what lies beyond
+// G in them is written as zero.
 // blockIdx.z is the matrix of a batch (pointers from the lists, sums of squares sumsq_stride apart).
 template <int DT>
-__global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, int cols,
+__global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, int cols, int rows_p, int cols_p,
                                                          int64_t ldg, const float* sumsq, int sumsq_stride,
                                                          float eps, PtrList Dl, int64_t ldd,
                                                          PtrList Tl, int64_t ldt,
@@ -165,21 +167,21 @@ __global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, i
         for (int e = 0; e < 8; ++e)
           o[e] = (c + e < cols) ? Elem<0>::st(as_bf16_value<DT>(src[e]) / denom) : (unsigned short)0;
       }
-      if (D) {
-        unsigned short* dst = D + (int64_t)r * ldd + c;
-        if (d_vec && c + 8 <= cols) {
-          union { uint4 v; unsigned short h[8]; } w;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) w.h[e] = o[e];
-          *reinterpret_cast<uint4*>(dst) = w.v;
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) if (c + e < cols) dst[e] = o[e];
-        }
-      }
     } else {
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] = 0;
+    }
+    if (D && r < rows_p) {
+      unsigned short* dst = D + (int64_t)r * ldd + c;
+      if (d_vec && c + 8 <= cols_p) {
+        union { uint4 v; unsigned short h[8]; } w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w.h[e] = o[e];
+        *reinterpret_cast<uint4*>(dst) = w.v;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) if (c + e < cols_p) dst[e] = o[e];
+      }
     }
     if (T) {
 #pragma unroll
@@ -192,16 +194,16 @@ __global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, i
   for (int pass = 0; pass < 2; ++pass) {
     const int lc = pass * 32 + (tid >> 3);   // column of G = row of T
     const int c = c0 + lc, r = r0 + ch * 8;
-    if (c < cols) {
+    if (c < cols_p) {
       unsigned short* dst = T + (int64_t)c * ldt + r;
       union { uint4 v; unsigned short h[8]; } w;
 #pragma unroll
       for (int e = 0; e < 8; ++e) w.h[e] = tile[(ch * 8 + e) * PITCH + lc];
-      if (t_vec && r + 8 <= rows) {
+      if (t_vec && r + 8 <= rows_p) {
         *reinterpret_cast<uint4*>(dst) = w.v;
       } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) if (r + e < rows) dst[e] = w.h[e];
+        for (int e = 0; e < 8; ++e) if (r + e < rows_p) dst[e] = w.h[e];
       }
     }
   }
@@ -209,7 +211,9 @@ __global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, i
 
 int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
                               const float* sumsq, int sumsq_stride, float eps, bf16_t* const* D, int64_t ldd,
-                              bf16_t* const* T, int64_t ldt, hipStream_t stream) {
+                              bf16_t* const* T, int64_t ldt, hipStream_t stream, int rows_p, int cols_p) {
+  if (rows_p < rows) rows_p = rows;
+  if (cols_p < cols) cols_p = cols;
   const int esz = dtype == 2 ? 4 : 2;
   int gv = (ldg * esz) % 16 == 0, dv = D != nullptr && ldd % 8 == 0, tv = T != nullptr && ldt % 8 == 0;
   PtrList gl = {}, dl = {}, tl = {};
@@ -219,8 +223,8 @@ int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int ro
     if (D) { dl.p[i] = D[i]; dv = dv && (reinterpret_cast<uintptr_t>(D[i]) & 15) == 0; }
     if (T) { tl.p[i] = T[i]; tv = tv && (reinterpret_cast<uintptr_t>(T[i]) & 15) == 0; }
   }
-  dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch), block(256);
-#define FM_SCALE(DT) hipLaunchKernelGGL(scale_cast_kernel<DT>, grid, block, 0, stream, gl, rows, cols, ldg, \
+  dim3 grid((unsigned)((cols_p + 63) / 64), (unsigned)((rows_p + 63) / 64), (unsigned)batch), block(256);
+#define FM_SCALE(DT) hipLaunchKernelGGL(scale_cast_kernel<DT>, grid, block, 0, stream, gl, rows, cols, rows_p, cols_p, ldg, \
                                         sumsq, sumsq_stride, eps, dl, ldd, tl, ldt, gv, dv, tv)
   if (dtype == 0) FM_SCALE(0);
   else if (dtype == 1) FM_SCALE(1);
@@ -233,7 +237,7 @@ int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
                       const float* sumsq, float eps, bf16_t* D, int64_t ldd, bf16_t* T, int64_t ldt,
                       hipStream_t stream) {
   return launch_scale_cast_batched(&G, 1, dtype, rows, cols, ldg, sumsq, 0, eps, D ? &D : nullptr, ldd,
-                                   T ? &T : nullptr, ldt, stream);
+                                   T ? &T : nullptr, ldt, stream, rows, cols);
 }
 
 // ---- momentum + Nesterov ------------------------------------------------------------------------
@@ -366,19 +370,7 @@ int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float
   return launch_weight_update_batched(&p, &u, 1, p_dtype, n, decay_mul, alpha, stream);
 }
 
-// ---- zero fill and 2-D copy, for the padded copies Newton-Schulz keeps of ragged matrices --------
-__global__ __launch_bounds__(256) void fill_zero_kernel(uint4* p, int64_t n16) {
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) p[i] = uint4{0u, 0u, 0u, 0u};
-}
-
-int launch_fill_zero(void* p, size_t bytes, hipStream_t stream) {   // p 16-byte aligned, bytes a multiple of 16
-  const int64_t n16 = (int64_t)(bytes / 16);
-  if (n16 == 0) return 0;
-  hipLaunchKernelGGL(fill_zero_kernel, dim3(stream_grid(n16)), dim3(256), 0, stream, static_cast<uint4*>(p), n16);
-  return (int)hipGetLastError();
-}
-
+// ---- 2-D copy with zero padding, for the whole-tile copies of matrices whose sides are not ---------
 // dst[b] (rows_d x cols_d, pitch ldd) = src[b] (rows x cols at src + b * bs_src, pitch lds) where
 // that exists and zero elsewhere, 16-bit elements.  A lane moves 8 consecutive elements of a row, as
 // one 16-byte access on a side that is aligned for it (`src_vec`, `dst_vec`) and element by element

@@ -137,7 +137,7 @@ int launch_sumsq_batched(const void* const* G, int batch, int dtype, int rows, i
                          float* out, int out_stride, float* partials, hipStream_t stream);
 int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
                               const float* sumsq, int sumsq_stride, float eps, bf16_t* const* D, int64_t ldd,
-                              bf16_t* const* T, int64_t ldt, hipStream_t stream);
+                              bf16_t* const* T, int64_t ldt, hipStream_t stream, int rows_p = 0, int cols_p = 0);
 int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, float* out,
                  float* partials, hipStream_t stream);
 int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
@@ -147,7 +147,6 @@ int launch_momentum_nesterov_batched(void* const* g, void* const* buf, int batch
                                      float w_buf, float w_nes, int nesterov, hipStream_t stream);
 int launch_weight_update_batched(void* const* p, const bf16_t* const* u, int batch, int p_dtype, int64_t n,
                                  float decay_mul, float alpha, hipStream_t stream);
-int launch_fill_zero(void* p, size_t bytes, hipStream_t stream);
 int launch_copy2d_batched(const bf16_t* src, int64_t lds, int64_t bs_src, bf16_t* const* dst, int64_t ldd,
                           int batch, int rows, int cols, int rows_d, int cols_d, hipStream_t stream);
 int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_buf, float w_nes,

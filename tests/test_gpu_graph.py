@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-# whole tiles, and sides that are not (zero-padded copies in the workspace: a fill kernel and copies)
+# whole tiles, and sides that are not (zero-padded copies in the workspace)
 @pytest.mark.parametrize("gshape,xshape", [((512, 1536), (768, 1024)), ((500, 1500), (700, 1000))])
 def test_graph_replays_match_eager(gshape, xshape):
     G = synthetic.gradient_like_bf16(gshape[0], gshape[1], 8, 41).to(DEV)
