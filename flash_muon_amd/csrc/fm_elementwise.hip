@@ -127,6 +127,18 @@ int launch_sumsq(const void* G, int dtype, int rows, int cols, int64_t ldg, floa
   return launch_sumsq_batched(&G, 1, dtype, rows, cols, ldg, out, 0, partials, stream);
 }
 
+// 16-byte accesses of data that is touched once per call: marked non-temporal, so that the stream
+// does not push anything else out of the caches
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld_stream(const void* p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return uint4{v.x, v.y, v.z, v.w};
+}
+__device__ __forceinline__ void st_stream(void* p, uint4 v) {
+  const u32x4_t w = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(w, reinterpret_cast<u32x4_t*>(p));
+}
+
 // ---- normalise, cast, transpose -----------------------------------------------------------------
 // One 64x64 tile of G per block: D gets the tile in place, T gets it transposed through LDS.
 // D is rows_p x cols_p and T cols_p x rows_p with rows_p >= rows, cols_p >= cols: what lies beyond
@@ -273,11 +285,11 @@ __global__ __launch_bounds__(256) void momentum_kernel(PtrList gl, PtrList bl, i
     uint4* b4 = reinterpret_cast<uint4*>(bv);
     for (int64_t i = t; i < nv; i += stride) {
       union { uint4 v; raw e[V]; } ug, ub;
-      ug.v = g4[i]; ub.v = b4[i];
+      ug.v = ld_stream(g4 + i); ub.v = ld_stream(b4 + i);
 #pragma unroll
       for (int e = 0; e < V; ++e) momentum_one<DT>(ug.e[e], ub.e[e], w_buf, w_nes, nesterov);
-      b4[i] = ub.v;
-      if (nesterov) g4[i] = ug.v;
+      st_stream(b4 + i, ub.v);
+      if (nesterov) st_stream(g4 + i, ug.v);
     }
     done = nv * V;
   }
@@ -331,16 +343,16 @@ __global__ __launch_bounds__(256) void weight_update_kernel(PtrList pl, PtrList 
     for (int64_t i = t; i < nv; i += stride) {
       union { uint4 v; unsigned short h[8]; } uu;
       union { uint4 v[sizeof(raw) / 2]; raw e[8]; } up;
-      uu.v = reinterpret_cast<const uint4*>(u)[i];
+      uu.v = ld_stream(reinterpret_cast<const uint4*>(u) + i);
 #pragma unroll
-      for (int q = 0; q < (int)sizeof(raw) / 2; ++q) up.v[q] = reinterpret_cast<uint4*>(pv)[i * (sizeof(raw) / 2) + q];
+      for (int q = 0; q < (int)sizeof(raw) / 2; ++q) up.v[q] = ld_stream(reinterpret_cast<uint4*>(pv) + i * (sizeof(raw) / 2) + q);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         float pf = Elem<DT>::ld(Elem<DT>::st(Elem<DT>::ld(up.e[e]) * decay_mul));
         up.e[e] = Elem<DT>::st(pf + alpha * Elem<0>::ld(uu.h[e]));
       }
 #pragma unroll
-      for (int q = 0; q < (int)sizeof(raw) / 2; ++q) reinterpret_cast<uint4*>(pv)[i * (sizeof(raw) / 2) + q] = up.v[q];
+      for (int q = 0; q < (int)sizeof(raw) / 2; ++q) st_stream(reinterpret_cast<uint4*>(pv) + i * (sizeof(raw) / 2) + q, up.v[q]);
     }
     done = nv * 8;
   }
