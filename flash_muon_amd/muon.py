@@ -180,9 +180,12 @@ class Muon(torch.optim.Optimizer):
                 assert p.is_cuda and g.is_cuda, "Muon parameters and gradients must be CUDA tensors"
                 buckets.setdefault((tuple(g.shape), g.dtype, p.dtype, g.device), []).append(p)
             for (_, _, _, dev), plist in buckets.items():
-                staging = self._staging_rows(update.numel(), min(self.batch, len(plist)), dev)
-                for i0 in range(0, len(plist), self.batch):
-                    chunk = plist[i0:i0 + self.batch]
+                # chunks of equal size (48 matrices go as 24 + 24, not 32 + 16): the launches of a small
+                # chunk leave most of the GPU idle, and those of a full one spill into a second round
+                per = -(-len(plist) // -(-len(plist) // self.batch))
+                staging = self._staging_rows(update.numel(), per, dev)
+                for i0 in range(0, len(plist), per):
+                    chunk = plist[i0:i0 + per]
                     n = len(chunk)
                     stream = _lib.stream_ptr(dev)
                     gcs, bufs = [], []
