@@ -203,6 +203,30 @@ def _extras(Xd, steps, warmup, torch):
     ex["muon_step_llama7b_ms"] = ms
     ex["muon_step_llama7b_useful_tflops"] = fl / ms / 1e9
     ex["muon_step_llama7b_frac_of_peak"] = fl / ms / 1e9 / PEAK_BF16_TFLOPS
+    del opt, params
+    torch.cuda.empty_cache()
+    # sides that are not whole tiles: both calls run on zero-padded copies in their workspace
+    Xr = synthetic.gaussian_bf16(4000, 4000, 4000).cuda()
+    ours_r = _time_gpu(lambda: matmul_transpose(Xr), 100, 30, torch)
+    ref_r = _time_gpu(lambda: torch.matmul(Xr, Xr.T), 100, 30, torch)
+    ex["xxt_4000_steady_ms"] = ours_r
+    ex["torch_xxt_4000_steady_ms"] = ref_r
+    ex["xxt_4000_steady_speedup_vs_torch"] = ref_r / ours_r
+    ns_r = _time_gpu(lambda: fast_newtonschulz(Xr, 5), 10, 3, torch)
+    ref_ns_r = _time_gpu(lambda: _torch_ns(Xr, 5, torch), 10, 3, torch)
+    ex["ns5_4000x4000_ms"] = ns_r
+    ex["torch_ns5_4000x4000_ms"] = ref_ns_r
+    ex["ns5_4000x4000_speedup_vs_torch"] = ref_ns_r / ns_r
+    del Xr
+    # Muon.step on a GPT-2-small-like set: 12 layers x (4 x 768^2, 3072x768, 768x3072)
+    params = []
+    for layer in range(12):
+        for (r, c) in ((768, 768),) * 4 + ((3072, 768), (768, 3072)):
+            p = torch.nn.Parameter((0.02 * torch.randn(r, c, generator=g, device="cuda", dtype=torch.float32)).bfloat16())
+            p.grad = (1e-3 * torch.randn(r, c, generator=g, device="cuda", dtype=torch.float32)).bfloat16()
+            params.append(p)
+    opt = Muon(params, lr=0.02, momentum=0.95, nesterov=True, rank=0, world_size=1)
+    ex["muon_step_gpt2_small_like_ms"] = _time_gpu(opt.step, 20, 5, torch)
     return ex
 
 
