@@ -69,8 +69,10 @@ def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
     if G.ndim > 2:
         flat = G.reshape(-1, G.size(-2), G.size(-1)).contiguous()
         out = torch.empty(flat.shape, dtype=torch.bfloat16, device=G.device)
-        for i0 in range(0, flat.size(0), MAX_BATCH):
-            n = min(MAX_BATCH, flat.size(0) - i0)
+        count = flat.size(0)
+        per = -(-count // -(-count // MAX_BATCH))   # chunks of equal size, as in Muon.step
+        for i0 in range(0, count, per):
+            n = min(per, count - i0)
             _newtonschulz_into([flat[i0 + i] for i in range(n)], [out[i0 + i] for i in range(n)], int(steps))
         return out.view(G.shape)
     if G.size(1) > 1 and G.stride(1) != 1 and G.stride(0) == 1 and G.stride(1) >= G.size(0):

@@ -143,7 +143,7 @@ def test_batched_matches_single_and_oracle(lib, rows, cols):
 
 def test_leading_dimensions_are_a_batch():
     """ndim > 2: every matrix of the leading dimensions is orthogonalised on its own (the norm of
-    muon.py:23 is over the last two dimensions), here 35 of them in chunks of 32 and 3."""
+    muon.py:23 is over the last two dimensions), here 35 of them in chunks of 18 and 17."""
     g = torch.Generator().manual_seed(31)
     G = (1e-3 * torch.randn(35, 96, 160, generator=g)).bfloat16().to(DEV)
     out = fast_newtonschulz(G, 5)
