@@ -1641,6 +1641,33 @@ static bool half_schedule_chosen(long long half_items, long long tiles, int nk, 
   return estimate_half_round(half_items, nk, grid) < estimate_whole_round(tiles, nk, auto_ksplit(tiles, nk, grid), grid);
 }
 
+// Few tiles (at most a sixteenth of the workgroups) can also run as 64x64 sub-tiles over the whole
+// k, 16 workgroups per tile, the way the tiles left after the last full round do: one launch, no
+// fp32 parts, and sixteen times the workgroups of whole tiles.  A sub-tile stage moves four times
+// the operand bytes per flop, so this pays up to about 64-80 k stages; beyond, the 128x128 tiles cut
+// along k win.  Measured on X X^T: 6.5 us + 0.205 us per stage (1024 x 1024 10, 1024 x 2048 13,
+// 1024 x 4096 20, 1024 x 8192 34 us); five Newton-Schulz steps at 1024^2 200 -> 176 us, 512 x 2048
+// 204 -> 170, 768^2 185 -> 160.
+static bool sub64_schedule_chosen(const GemmArgs& a, long long tiles, int nk, int grid) {
+  const long long ns = knob(kKnobNoSub64);       // 1: never; 0: whenever it fits; left alone: by the estimate below
+  if (ns > 0 || tiles < 1 || tiles * 16 > grid) return false;
+  if (ns == 0) return true;
+  if (knob(kKnobKsplit) >= 0 || knob(kKnobHalf) >= 0 || knob(kKnobFastMinUnits) >= 0) return false;
+  const long long tm = a.Ma / BM, tn = a.Nb / BN, nb = a.batch < 1 ? 1 : a.batch;
+  const double t_sub = nk * 0.205 + 6.5 + (a.E ? 2.0 : 0.0);
+  const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * nb;
+  double t_best = estimate_mid(small_tiles, nk, grid, a.E != nullptr);
+  const int ksplit = auto_ksplit(tiles, nk, grid);
+  const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
+  if (t_large < t_best) t_best = t_large;
+  const long long half_items = (a.symmetric ? tm * tm : 2 * tm * tn) * nb;
+  if (half_schedule_chosen(half_items, tiles, nk, grid)) {
+    const double t_half = estimate_half_round(half_items, nk, grid);
+    if (t_half < t_best) t_best = t_half;
+  }
+  return t_sub < t_best;
+}
+
 bool gemm_fast_eligible(const GemmArgs& a) {
   if (!tiled_dma_eligible(a, BM)) return false;
   // the write-out reads the epilogue operand transposed, 16 bytes at a time
@@ -1656,6 +1683,7 @@ bool gemm_fast_eligible(const GemmArgs& a) {
   // microseconds from the measured cost of a k stage and of a tile's epilogue on each path.
   const int cus = cu_count() < kMaxGrid ? cu_count() : kMaxGrid;
   if (tiles > cus) return true;
+  if (sub64_schedule_chosen(a, tiles, nk, cus)) return true;
   const int ksplit = auto_ksplit(tiles, nk, cus);
   const double t_large = (nk / ksplit) * 1.45 + 15.0 + (ksplit > 1 ? 25.0 : 0.0);
   const long long small_tiles = (a.symmetric ? 2 * tm * (2 * tm + 1) / 2 : 4 * tm * tn) * (a.batch < 1 ? 1 : a.batch);
@@ -1733,7 +1761,16 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   const long long kg = knob(kKnobGrid);
   if (kg > 0 && kg < grid) grid = (int)kg;
   const long long half_items = a.symmetric ? (long long)a.tiles_m * a.tiles_m * a.batch : 2LL * a.num_tiles;   // a diagonal tile is one item
-  if (half_items < (1LL << 30) && half_schedule_chosen(half_items, a.num_tiles, f.nk, grid)) {   // 128x256 half tiles, whole, in rounds
+  if (sub64_schedule_chosen(a, a.num_tiles, f.nk, grid)) {   // every tile as 16 sub-tiles of 64x64, one workgroup each
+    f.grid = a.num_tiles * 16;
+    f.ksplit = 1;
+    f.rounds = 0;
+    f.rem = a.num_tiles;
+    f.split = 1;
+    f.sub64 = 1;
+    f.tail_slot0 = 0;
+    f.reduce_tile0 = a.num_tiles;
+  } else if (half_items < (1LL << 30) && half_schedule_chosen(half_items, a.num_tiles, f.nk, grid)) {   // 128x256 half tiles, whole, in rounds
     const int items = (int)half_items;
     if (grid > items) grid = items;
     f.half = 1;

@@ -66,7 +66,9 @@ enum fm_knob {
   FM_KNOB_FAST_MIN_UNITS = 2,  /* take the 256x256 schedule when tiles * k-stages >= this (0: whenever the shape allows) */
   FM_KNOB_NO_MID = 3,          /* 1: never take the 128x128 copy-fed schedule */
   FM_KNOB_NO_SUB64 = 4,        /* 1: cut the tiles left after the last full round along k (fp32 parts, second
-                                  kernel) even where 64x64 sub-tiles over the whole k would do */
+                                  kernel) even where 64x64 sub-tiles over the whole k would do, and never run
+                                  a whole product on such sub-tiles; 0: run every product of at most a
+                                  sixteenth as many 256x256 tiles as workgroups on them (by estimate otherwise) */
   FM_KNOB_HALF = 5             /* 1: always, 0: never run the 256x256 schedule on 128x256 half tiles (taken by
                                   itself when all of them fit into one round of workgroups) */
 };
