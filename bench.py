@@ -23,11 +23,23 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 DIM = 8192
-# L2-miss traffic of one 8192^2 call (a single kernel), from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads for a 128 MiB device copy (FETCH_SIZE reads
-# half of the copied bytes there, WRITE_SIZE all of them): 508.3e3 KiB * 2.0 fetched + 131.1e3 KiB
-# written.  The commands and the raw readings are in profiles/syrk_bf16_8192_traffic.md.
-TRAFFIC_BYTES = int(508.3e3 * 1024 * 2.0 + 131.1e3 * 1024 * 1.0)
+# L2-miss traffic of one 8192^2 call (a single kernel) is not measured by this script: it comes from
+# rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of it, each scaled by what the same counter reads
+# for a 128 MiB device copy.  The commands, the raw readings and the line
+# `traffic_bytes_per_call: N` that is read here are in this file:
+TRAFFIC_FILE = os.path.join("profiles", "syrk_bf16_8192_traffic.md")
+
+
+def _traffic_bytes():
+    """(bytes per call, where the figure comes from), or (None, why not)."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            for ln in f:
+                if ln.startswith("traffic_bytes_per_call:"):
+                    return int(float(ln.split(":", 1)[1].split()[0])), "constant from %s (rocprofv3 counters, not this run)" % TRAFFIC_FILE
+    except OSError:
+        pass
+    return None, "%s holds no traffic_bytes_per_call line" % TRAFFIC_FILE
 
 
 def _time_gpu(fn, steps, warmup, torch):
@@ -44,11 +56,38 @@ def _time_gpu(fn, steps, warmup, torch):
     return start.elapsed_time(end) / steps   # ms per call
 
 
+def _median(v):
+    v = sorted(v)
+    return v[len(v) // 2] if len(v) % 2 else 0.5 * (v[len(v) // 2 - 1] + v[len(v) // 2])
+
+
+def _interleaved(fns, calls, blocks, warm, torch):
+    """Time the functions of `fns` (name -> callable) in the same phase of the chip's power management:
+    `warm` calls of each, then `blocks` rounds in which every function in turn is timed over `calls`
+    calls (the reference times its functions back to back per size, benchmark.py:66-80).  Returns
+    name -> (median ms per call over the blocks, the blocks)."""
+    for fn in fns.values():
+        for _ in range(warm):
+            fn()
+    torch.cuda.synchronize()
+    t = {k: [] for k in fns}
+    for _ in range(blocks):
+        for k, fn in fns.items():
+            t[k].append(_time_gpu(fn, calls, 0, torch))
+    return {k: (_median(v), v) for k, v in t.items()}
+
+
 def _mfma_probe(torch):
     """Sustained rate and clock of MFMA-only work (fm_probe_mfma_peak), on zeros and on N(0,1) bf16
     operands: about 150 ms of back-to-back launches each, the second half timed."""
-    from flash_muon_amd import _lib
-    lib = _lib.load()
+    import ctypes
+    from flash_muon_amd import _lib, build
+    if not os.path.exists(build.PROBE_LIB_PATH):
+        build.build()
+    lib = ctypes.CDLL(build.PROBE_LIB_PATH)   # the probe is not part of the product library
+    vp = ctypes.c_void_p
+    lib.fm_probe_mfma_peak.restype = ctypes.c_int
+    lib.fm_probe_mfma_peak.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
     blocks, iters, launches = 256, 256, 480
     sink = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
     clocks = torch.zeros(blocks * 2, dtype=torch.int64, device="cuda")
@@ -142,50 +181,37 @@ def _torch_ns(G, steps, torch):
 def _extras(Xd, steps, warmup, torch):
     from flash_muon_amd import Muon, fast_newtonschulz, synthetic
     ex = {}
-    # vendor GEMM for the same product, both BLAS back ends torch can select
-    for name, pref in (("rocblas", "cublas"), ("hipblaslt", "cublaslt")):
-        try:
-            torch.backends.cuda.preferred_blas_library(pref)
-            ex["torch_xxt_%s_ms" % name] = _time_gpu(lambda: torch.matmul(Xd, Xd.T), steps, warmup, torch)
-        except Exception as e:   # report, never hide
-            ex["torch_xxt_%s_ms" % name] = "failed: %s" % e
-    torch.backends.cuda.preferred_blas_library("default")
-    # the smaller sizes of the square sweep (seed = dim; 1024 is the CPU-sized case, seed 0)
+    # The smaller sizes of the square sweep (seed = dim; 1024 is the CPU-sized case, seed 0) and a wide
+    # input with few output tiles and a long k.  Every speed-up is a ratio of medians of blocks that
+    # alternate between the two functions after a warm-up of both (six blocks of 50 calls each), so
+    # that both are timed in the same state of the chip; the reference's own protocol (W + K calls
+    # of one function, then of the other, benchmark.py:66-80) is reported as times only.
     from flash_muon_amd import matmul_transpose
-    for dim, seed in ((1024, 0), (2048, 2048), (4096, 4096)):
-        Xs = synthetic.gaussian_bf16(dim, dim, seed).cuda()
-        ours = _time_gpu(lambda: matmul_transpose(Xs), steps, warmup, torch)
-        ref = _time_gpu(lambda: torch.matmul(Xs, Xs.T), steps, warmup, torch)
-        ex["xxt_%d_ms" % dim] = ours
-        ex["xxt_%d_useful_tflops" % dim] = synthetic.syrk_useful_flop(dim, dim) / ours / 1e9
-        ex["torch_xxt_%d_ms" % dim] = ref
-        ex["xxt_%d_speedup_vs_torch" % dim] = ref / ours
-        # W + K calls of these sizes last a few milliseconds and fall into the power-management
-        # transient after idle; the same pair once more over 100 + 200 calls each
-        ours_s = _time_gpu(lambda: matmul_transpose(Xs), 200, 100, torch)
-        ref_s = _time_gpu(lambda: torch.matmul(Xs, Xs.T), 200, 100, torch)
-        ex["xxt_%d_steady_ms" % dim] = ours_s
-        ex["torch_xxt_%d_steady_ms" % dim] = ref_s
-        ex["xxt_%d_steady_speedup_vs_torch" % dim] = ref_s / ours_s
+    for rows, cols, seed in ((1024, 1024, 0), (2048, 2048, 2048), (4096, 4096, 4096), (1024, 8192, 1024)):
+        Xs = synthetic.gaussian_bf16(rows, cols, seed).cuda()
+        tag = "%d" % rows if rows == cols else "%dx%d" % (rows, cols)
+        if rows == cols:
+            ex["xxt_%s_ms" % tag] = _time_gpu(lambda: matmul_transpose(Xs), steps, warmup, torch)
+            ex["torch_xxt_%s_ms" % tag] = _time_gpu(lambda: torch.matmul(Xs, Xs.T), steps, warmup, torch)
+        r = _interleaved({"ours": lambda: matmul_transpose(Xs), "torch": lambda: torch.matmul(Xs, Xs.T)},
+                         50, 6, 100, torch)
+        ex["xxt_%s_steady_ms" % tag] = r["ours"][0]
+        ex["torch_xxt_%s_steady_ms" % tag] = r["torch"][0]
+        ex["xxt_%s_steady_speedup_vs_torch" % tag] = r["torch"][0] / r["ours"][0]
+        ex["xxt_%s_steady_useful_tflops" % tag] = synthetic.syrk_useful_flop(rows, cols) / r["ours"][0] / 1e9
         del Xs
-    # a wide input with few output tiles and a long k (cut along k on the 128x128 path), steady state
-    Xw = synthetic.gaussian_bf16(1024, 8192, 1024).cuda()
-    ours_w = _time_gpu(lambda: matmul_transpose(Xw), 200, 100, torch)
-    ref_w = _time_gpu(lambda: torch.matmul(Xw, Xw.T), 200, 100, torch)
-    ex["xxt_1024x8192_steady_ms"] = ours_w
-    ex["torch_xxt_1024x8192_steady_ms"] = ref_w
-    ex["xxt_1024x8192_steady_speedup_vs_torch"] = ref_w / ours_w
-    del Xw
     # fast_newtonschulz(5) on the gradient-like inputs of the rectangular and the square case
     # (noise of std 1e-3 plus a rank-r spike, Frobenius-normalised; generated on the CPU from the
     # seed so that the CPU oracle sees the same bits)
     for rows, cols, rank, seed in ((8192, 8192, 16, 4), (4096, 16384, 8, 3)):
         G = synthetic.gradient_like_bf16(rows, cols, rank, seed).cuda()
-        ms = _time_gpu(lambda: fast_newtonschulz(G, 5), 10, 3, torch)
+        r = _interleaved({"ours": lambda: fast_newtonschulz(G, 5), "torch": lambda: _torch_ns(G, 5, torch)},
+                         5, 3, 3, torch)
+        ms, ref_ms = r["ours"][0], r["torch"][0]
         fl = synthetic.ns_useful_flop(rows, cols, 5)
         ex["ns5_%dx%d_ms" % (rows, cols)] = ms
         ex["ns5_%dx%d_useful_tflops" % (rows, cols)] = fl / ms / 1e9
-        ref_ms = _time_gpu(lambda: _torch_ns(G, 5, torch), 10, 3, torch)
+        ex["ns5_%dx%d_frac_of_peak" % (rows, cols)] = fl / ms / 1e9 / PEAK_BF16_TFLOPS
         ex["torch_ns5_%dx%d_ms" % (rows, cols)] = ref_ms
         ex["ns5_%dx%d_speedup_vs_torch" % (rows, cols)] = ref_ms / ms
         del G
@@ -198,22 +224,56 @@ def _extras(Xd, steps, warmup, torch):
             p.grad = (1e-3 * torch.randn(r, c, generator=g, device="cuda", dtype=torch.float32)).bfloat16()
             params.append(p)
     opt = Muon(params, lr=0.02, momentum=0.95, nesterov=True, rank=0, world_size=1)
-    ms = _time_gpu(opt.step, 3, 1, torch)
+    # Twins of two parameters, stepped one matrix per launch afterwards: the last 4096^2 matrix (whose
+    # update the group's buffer still holds after a step) and an 11008 x 4096 one.
+    last_sq = max(i for i, p in enumerate(params) if tuple(p.shape) == (4096, 4096))
+    tall = next(i for i, p in enumerate(params) if tuple(p.shape) == (11008, 4096))
+    twins = []
+    for i in (last_sq, tall):
+        q = torch.nn.Parameter(params[i].detach().clone())
+        q.grad = params[i].grad.clone()
+        twins.append(q)
+    nsteps = 4   # one warm-up and three timed steps
+    ms = _time_gpu(opt.step, nsteps - 1, 1, torch)
     fl = sum(synthetic.ns_useful_flop(r, c, 5) for (r, c) in synthetic.LLAMA7B_LAYER_SHAPES) * 32
     ex["muon_step_llama7b_ms"] = ms
     ex["muon_step_llama7b_useful_tflops"] = fl / ms / 1e9
     ex["muon_step_llama7b_frac_of_peak"] = fl / ms / 1e9 / PEAK_BF16_TFLOPS
-    del opt, params
+    # what was timed is looked at: every parameter finite, and the two twins, stepped the same number
+    # of times one matrix per launch, end where their originals did (bf16 parameters: the two runs
+    # differ in fp32 summation order, which flips the rounding of a few elements of a step)
+    for p in params:
+        assert bool(torch.isfinite(p).all()), "Muon.step left a parameter that is not finite"
+    for q, i, name in ((twins[0], last_sq, "4096x4096"), (twins[1], tall, "11008x4096")):
+        q0 = q.detach().clone()
+        topt = Muon([q], lr=0.02, momentum=0.95, nesterov=True, rank=0, world_size=1, batch=1)
+        for _ in range(nsteps):
+            topt.step()
+        moved = (params[i].detach().float() - q0.float())
+        diff = (params[i].detach().float() - q.detach().float())
+        rel = float(diff.norm() / moved.norm())
+        ex["muon_step_llama7b_%s_vs_one_per_launch_rel_fro" % name] = rel
+        assert rel < 0.1, "Muon.step at 32 per launch and at 1 per launch moved a %s parameter differently: %g" % (name, rel)
+        assert torch.equal(q.grad, params[i].grad), "momentum / Nesterov state differs"
+        if i == last_sq:   # the orthogonalised update itself, as the last step left it in the group's buffer
+            ub = [g["update_buffer"][0] for g in opt.param_groups if g["params"][-1] is params[i]]
+            if ub:
+                tu = topt.param_groups[0]["update_buffer"][0].float()
+                rel_u = float((ub[0].float() - tu).norm() / tu.norm())
+                ex["muon_step_llama7b_update_vs_one_per_launch_rel_fro"] = rel_u
+                assert rel_u < 6e-3, "update of the last 4096^2 parameter differs from the one-per-launch one: %g" % rel_u
+        del topt
+    del opt, params, twins
     torch.cuda.empty_cache()
     # sides that are not whole tiles: both calls run on zero-padded copies in their workspace
     Xr = synthetic.gaussian_bf16(4000, 4000, 4000).cuda()
-    ours_r = _time_gpu(lambda: matmul_transpose(Xr), 100, 30, torch)
-    ref_r = _time_gpu(lambda: torch.matmul(Xr, Xr.T), 100, 30, torch)
+    r = _interleaved({"ours": lambda: matmul_transpose(Xr), "torch": lambda: torch.matmul(Xr, Xr.T)}, 50, 4, 50, torch)
+    ours_r, ref_r = r["ours"][0], r["torch"][0]
     ex["xxt_4000_steady_ms"] = ours_r
     ex["torch_xxt_4000_steady_ms"] = ref_r
     ex["xxt_4000_steady_speedup_vs_torch"] = ref_r / ours_r
-    ns_r = _time_gpu(lambda: fast_newtonschulz(Xr, 5), 10, 3, torch)
-    ref_ns_r = _time_gpu(lambda: _torch_ns(Xr, 5, torch), 10, 3, torch)
+    r = _interleaved({"ours": lambda: fast_newtonschulz(Xr, 5), "torch": lambda: _torch_ns(Xr, 5, torch)}, 5, 3, 3, torch)
+    ns_r, ref_ns_r = r["ours"][0], r["torch"][0]
     ex["ns5_4000x4000_ms"] = ns_r
     ex["torch_ns5_4000x4000_ms"] = ref_ns_r
     ex["ns5_4000x4000_speedup_vs_torch"] = ref_ns_r / ns_r
@@ -243,6 +303,9 @@ def main():
     ap.add_argument("--mfma-probe", action="store_true",
                     help="only run the MFMA-only loop on zeros and on N(0,1) operands and print its sustained "
                          "TFLOP/s and shader clock: the ceiling the power cap sets for matrix work")
+    ap.add_argument("--vendor-gemm", choices=("rocblas", "hipblaslt"),
+                    help="only run W + K calls of torch.matmul(X, X.T) on the 8192^2 input with that BLAS back "
+                         "end and print their time: the vendor kernel by itself, for counter runs beside ours")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 128 MiB device-to-device copy, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counter readings are scaled by")
@@ -265,6 +328,12 @@ def main():
 
     X = synthetic.gaussian_bf16(DIM, DIM, DIM)
     Xd = X.cuda()
+    if args.vendor_gemm:
+        torch.backends.cuda.preferred_blas_library({"rocblas": "cublas", "hipblaslt": "cublaslt"}[args.vendor_gemm])
+        ms = _time_gpu(lambda: torch.matmul(Xd, Xd.T), args.steps, args.warmup, torch)
+        print(json.dumps({"vendor_gemm": args.vendor_gemm, "ms_per_call": ms, "steps": args.steps,
+                          "executed_tflops": 2.0 * DIM ** 3 / ms / 1e9}))
+        return
     Y = torch.empty(DIM, DIM, dtype=torch.bfloat16, device="cuda")
     torch.cuda.empty_cache()
     # The same W + K calls straight after the idle time of the input generation: the power
@@ -273,8 +342,26 @@ def main():
     # which is taken after the other timings below have run.
     cold_ms = _time_gpu(lambda: matmul_transpose_assign(Xd, Y), args.steps, args.warmup, torch)
     ex = None
+    vendor = {}
     if not args.no_extras:
         ex = _extras(Xd, args.steps, args.warmup, torch)
+        # The vendor GEMM for the same product, with both BLAS back ends torch can select, in the same
+        # phase as this library's call: after 100 calls of ours, six rounds of 20 calls of each of
+        # the three in turn.  Every speed-up over the vendor below is a ratio of these medians.
+        def blas(pref):
+            def f():
+                torch.backends.cuda.preferred_blas_library(pref)
+                return torch.matmul(Xd, Xd.T)
+            return f
+        try:
+            vendor = _interleaved({"ours": lambda: matmul_transpose_assign(Xd, Y), "rocblas": blas("cublas"),
+                                   "hipblaslt": blas("cublaslt")}, 20, 6, 34, torch)
+        except Exception as e:   # report, never hide
+            vendor = {"error": "%s" % e}
+        torch.backends.cuda.preferred_blas_library("default")
+    # sustained: 200 calls after 100 (a quarter of a second of nothing but this kernel)
+    steady_ms = _time_gpu(lambda: matmul_transpose_assign(Xd, Y), 200, 100, torch)
+    # the headline, straight after that sustained run
     ms = _time_gpu(lambda: matmul_transpose_assign(Xd, Y), args.steps, args.warmup, torch)
     assert torch.equal(Y, Y.T), "output is not symmetric"
     # the spread of the timed region, in blocks of 5 calls
@@ -286,6 +373,7 @@ def main():
 
     useful = synthetic.syrk_useful_flop(DIM, DIM)
     tflops = useful / ms / 1e9
+    traffic, traffic_source = _traffic_bytes()
     line = {
         "metric": "matmul_transpose useful TFLOP/s at 8192x8192 bf16",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -295,17 +383,25 @@ def main():
                    "M": DIM, "K": DIM},
         "effective_tflops": 2.0 * DIM * DIM * DIM / ms / 1e9,
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": TRAFFIC_BYTES,
+                     "frac": tflops / PEAK_BF16_TFLOPS, "traffic": traffic,
+                     "traffic_source": traffic_source,
                      "flop_per_launch": useful, "kernel": "gemm_nt_rounds_kernel"},
     }
     if not args.no_cpu:
         line["cpu_baseline"] = _cpu_baseline(X, torch, ns=not args.no_extras, full=args.cpu_full)
     if ex is None:
         ex = {}
-    else:
-        for k in ("torch_xxt_rocblas_ms", "torch_xxt_hipblaslt_ms"):
-            if isinstance(ex.get(k), float):
-                ex[k.replace("_ms", "_speedup")] = ex[k] / ms
+    if "error" in vendor:
+        ex["torch_xxt_vendor"] = "failed: " + vendor["error"]
+    elif vendor:
+        ex["xxt_8192_same_phase_ms"] = vendor["ours"][0]
+        ex["xxt_8192_same_phase_blocks_ms"] = vendor["ours"][1]
+        for name in ("rocblas", "hipblaslt"):
+            ex["torch_xxt_%s_ms" % name] = vendor[name][0]
+            ex["torch_xxt_%s_blocks_ms" % name] = vendor[name][1]
+            ex["torch_xxt_%s_speedup" % name] = vendor[name][0] / vendor["ours"][0]
+    ex["xxt_8192_steady_ms"] = steady_ms
+    ex["xxt_8192_steady_frac_of_peak"] = useful / steady_ms / 1e9 / PEAK_BF16_TFLOPS
     ex["ms_per_step_first_calls_after_idle"] = cold_ms
     ex["ms_per_step_blocks_of_5_after"] = blocks
     ex["ms_per_step_best_block"] = min(blocks)

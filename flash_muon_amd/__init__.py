@@ -5,5 +5,6 @@ The four public names and their signatures are those of the reference package
 """
 from .matmul_transpose import matmul_transpose, matmul_transpose_assign
 from .muon import fast_newtonschulz, Muon
+from ._lib import release_workspaces   # not in the reference: drops the cached GEMM scratch
 
 __all__ = ["matmul_transpose", "matmul_transpose_assign", "fast_newtonschulz", "Muon"]

@@ -15,7 +15,7 @@ FM_OK = 0
 FM_ERR_STRIDE = 3
 FM_ERR_ALIAS = 5
 # fm_knob values
-FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID, FM_KNOB_NO_SUB64, FM_KNOB_HALF = 0, 1, 2, 3, 4, 5
+FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID, FM_KNOB_NO_SUB64, FM_KNOB_HALF, FM_KNOB_DIAG_LAST = 0, 1, 2, 3, 4, 5, 6
 FM_BF16, FM_F16, FM_F32 = 0, 1, 2
 
 _DTYPE_CODE = {torch.bfloat16: FM_BF16, torch.float16: FM_F16, torch.float32: FM_F32}
@@ -50,7 +50,6 @@ SIGNATURES = {
     "fm_weight_update": (_i32, [_vp, _i32, _vp, _i64, _f32, _f32, _vp]),
     "fm_momentum_nesterov_batched": (_i32, [_vp, _vp, _i32, _i32, _i64, _f32, _f32, _i32, _vp]),
     "fm_weight_update_batched": (_i32, [_vp, _i32, _vp, _i32, _i64, _f32, _f32, _vp]),
-    "fm_probe_mfma_peak": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp]),
 }
 
 _lib = None
@@ -146,3 +145,11 @@ def gemm_workspace(nbytes, device, stream=None):
     if ws is None or ws.numel() < nbytes:
         ws = _gemm_ws[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)
     return ws, ws.numel()
+
+
+def release_workspaces():
+    """Give the cached scratch of the single GEMM-shaped calls back to torch's allocator.  One
+    tensor per (device, stream) is kept and only ever grows (up to about 256 MiB each); call this after
+    the last matmul_transpose on streams that will not be used again, or to drop a block that a call
+    under graph capture took from the graph's private pool.  Not while such calls are in flight."""
+    _gemm_ws.clear()

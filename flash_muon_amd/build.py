@@ -13,7 +13,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJDIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libflashmuon_hip.so")
-SOURCES = ["fm_gemm.hip", "fm_gemm_fast.hip", "fm_elementwise.hip", "fm_api.hip", "fm_probe.hip"]
+SOURCES = ["fm_gemm.hip", "fm_gemm_fast.hip", "fm_elementwise.hip", "fm_api.hip"]
+# a measurement aid (MFMA-only loop) that only `bench.py --mfma-probe` loads; a library of its own
+PROBE_LIB_PATH = os.path.join(HERE, "libflashmuon_probe.so")
+PROBE_SOURCES = [os.path.join("probe", "fm_probe.hip")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -25,7 +28,7 @@ FLAGS = [
 
 
 def _compile(src):
-    obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
+    obj = os.path.join(OBJDIR, os.path.splitext(os.path.basename(src))[0] + ".o")
     cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # hipcc's host pass prints that it ignores the packed-fp32 target feature; drop that line
@@ -37,18 +40,23 @@ def _compile(src):
     return obj
 
 
-def build(verbose=True):
-    os.makedirs(OBJDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    tmp = LIB_PATH + ".tmp"
+def _link(objs, path):
+    tmp = path + ".tmp"
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s" % r.stderr)
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, path)
+
+
+def build(verbose=True):
+    os.makedirs(OBJDIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=5) as ex:
+        objs = list(ex.map(_compile, SOURCES + PROBE_SOURCES))
+    _link(objs[:len(SOURCES)], LIB_PATH)
+    _link(objs[len(SOURCES):], PROBE_LIB_PATH)
     if verbose:
-        print("built", LIB_PATH)
+        print("built", LIB_PATH, "and", PROBE_LIB_PATH)
     return LIB_PATH
 
 

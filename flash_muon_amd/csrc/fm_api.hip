@@ -135,14 +135,15 @@ int fm_set_knob(int which, long long value) { return set_knob(which, value) == 0
 
 // X * X^T of a matrix whose sides are not whole 128-tiles, through zero-padded copies: X padded in
 // the workspace, the product of that on the tiled paths into a padded Y beside it, and the M x M
-// part copied out.  Pays from about a million elements of X on (below that the general path's single
-// launch wins); 16-bit elements only.
+// part copied out.  Taken from 65536 elements of X on (below that the general path's single launch
+// wins); 16-bit elements only.  The tiled paths need whole 128-row tiles and whole 64-wide k stages,
+// so a shape that has both is left alone and k is padded to a multiple of 64 only.
 struct SyrkPad { int Mp, Kp; size_t x, y, gemm, total; };
 constexpr int64_t kSyrkPadMinElems = 256 * 256;
 static bool syrk_pad_layout(int M, int K, SyrkPad* p) {
-  if (M <= 0 || K <= 0 || (M % 128 == 0 && K % 128 == 0) || (int64_t)M * K < kSyrkPadMinElems) return false;
+  if (M <= 0 || K <= 0 || (M % 128 == 0 && K % 64 == 0) || (int64_t)M * K < kSyrkPadMinElems) return false;
   p->Mp = ns_pad(M);
-  p->Kp = (K + 127) / 128 * 128;
+  p->Kp = (K + 63) / 64 * 64;
   p->x = 0;
   p->y = align_up((size_t)p->Mp * p->Kp * 2, 256);
   p->gemm = p->y + align_up((size_t)p->Mp * p->Mp * 2, 256);
@@ -223,7 +224,7 @@ int fm_syrk_bf16_static(const void* X, int64_t ldx, void* Y, int64_t ldy_row, in
   void* scratch = nullptr;
   const int rc = static_scratch(&scratch);
   if (rc != FM_OK) return rc;
-  // always the schedules of fm_syrk_bf16 with a workspace of fm_gemm_workspace_bytes(M, M), bit for bit
+  // the schedules, and the bits, of fm_syrk_bf16 given a workspace of these 64 MiB (no padded copies)
   return syrk_impl(X, ldx, Y, ldy_row, ldy_col, M, K, scratch, kStaticScratchBytes, stream, kElemBf16, false);
 }
 

@@ -5,9 +5,13 @@
 // Schedule.  One workgroup per CU.  Tiles are taken in rounds of `grid` whole tiles: all workgroups
 // start a tile together and walk k in step, so the workgroups of one XCD, which hold a compact
 // block of tiles, find each other's operand panels in their shared L2.  What is left after the
-// last full round (fewer tiles than workgroups) is cut along k into `split` parts per tile, one
-// part per workgroup, so that the last round is as short as its share of the work; the parts go to
-// memory as fp32 and a second, small kernel adds them in part order and runs the epilogue.
+// last full round (fewer tiles than workgroups) is cut so that the last round is as short as its
+// share of the work: in space, into 64x64 sub-tiles over the whole k, when at most a sixteenth as
+// many tiles as workgroups are left (nothing is added up afterwards; of a symmetric product the
+// tiles left are diagonal ones); otherwise along k into `split` parts per tile, one part per
+// workgroup, which go to memory as fp32 and are added in part order by a second, small kernel that
+// also runs the epilogue.  A product whose 128x256 half tiles fit into one round runs on those, and
+// one of at most 16 tiles may run on sub-tiles altogether.
 #include "fm_internal.h"
 
 #include <type_traits>
@@ -761,16 +765,37 @@ __device__ __forceinline__ void tile_at(const GemmArgs& g, int pos, int& b, int&
     b = pos / per_matrix;
     pos -= b * per_matrix;
   }
+  // the last `diag_last` diagonal tiles of a symmetric product stand at the end of the order
+  const int d0 = g.tiles_m - g.diag_last;   // first of them (tiles_m without any)
+  if (g.diag_last > 0 && pos >= g.num_tiles - g.diag_last) {
+    ti = tj = d0 + (pos - (g.num_tiles - g.diag_last));
+    return;
+  }
   const int nbm = (g.tiles_m + SB - 1) / SB, nbn = (g.tiles_n + SB - 1) / SB;
   for (int I = 0; I < nbm; ++I) {
     const int rows = (g.tiles_m - I * SB) < SB ? (g.tiles_m - I * SB) : SB;
     for (int J = g.symmetric ? I : 0; J < nbn; ++J) {
       const int cols = (g.tiles_n - J * SB) < SB ? (g.tiles_n - J * SB) : SB;
       const bool tri = g.symmetric && I == J;
-      const int cnt = tri ? rows * (rows + 1) / 2 : rows * cols;
+      // diagonal tiles of this block that stand at the end instead
+      int gone = 0;
+      if (tri && g.diag_last > 0) {
+        gone = I * SB + rows - d0;
+        gone = gone < 0 ? 0 : gone > rows ? rows : gone;
+      }
+      const int cnt = tri ? rows * (rows + 1) / 2 - gone : rows * cols;
       if (pos < cnt) {
         int a, b;
-        if (tri) { tri_decode(pos, rows, a, b); } else { a = pos / cols; b = pos - a * cols; }
+        if (!tri) { a = pos / cols; b = pos - a * cols; }
+        else if (gone == 0) { tri_decode(pos, rows, a, b); }
+        else {   // row a of the triangle holds rows - a tiles, one fewer without its diagonal tile
+          for (a = 0; a < rows - 1; ++a) {
+            const int in_row = rows - a - (I * SB + a >= d0 ? 1 : 0);
+            if (pos < in_row) break;
+            pos -= in_row;
+          }
+          b = a + pos + (I * SB + a >= d0 ? 1 : 0);
+        }
         ti = I * SB + a;
         tj = J * SB + b;
         return;
@@ -1057,8 +1082,8 @@ __device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, in
 // MODE: how whole tiles are written out (see epilogue_regs); chosen by the host from E and beta
 template <bool F16, int MODE, int NI>
 __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
-  // two operand stages (A0 B0 A1 B1, 32 KiB each) during the main loop, the accumulator staging of
-  // the four waves afterwards
+  // the operand ring during the main loop (five slots of 32 KiB: A0 A1 B0 B1 A2), the staging of
+  // the four waves' write-out afterwards
   __shared__ __align__(1024) unsigned char smem[SMEM_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1783,6 +1808,11 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
     f.tail_slot0 = 0;
     f.reduce_tile0 = a.num_tiles;
   }
+  // Sub-tiles left over from a symmetric product: let them be diagonal tiles.  Such a tile needs one
+  // operand panel where another needs two (the last round is bound by what the L2s fetch), and 10 of
+  // its 16 sub-tiles are distinct.  The bits are those of any other order.
+  if (f.sub64 && f.rounds > 0 && a.symmetric && a.batch == 1 && f.rem <= a.tiles_m && knob(kKnobDiagLast) != 0)
+    f.g.diag_last = f.rem;
   f.partials = static_cast<float*>(ws);
   if (f.half) {
     if (a.elem == kElemF16) hipLaunchKernelGGL((gemm_nt_rounds_kernel<true, 0, 2>), dim3(f.grid), dim3(256), 0, stream, f);

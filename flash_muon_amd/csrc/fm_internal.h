@@ -21,7 +21,7 @@ constexpr int kErrWorkspace = -2;     // the schedule needs more partial-tile sl
 // Tuning knobs (fm_set_knob, include/flashmuon.h); the FLASHMUON_* environment variables of the same
 // names give their initial values, read once when the library is first used.  A negative value
 // means "decide automatically".
-constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobNoSub64 = 4, kKnobHalf = 5, kKnobCount = 6;
+constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobNoSub64 = 4, kKnobHalf = 5, kKnobDiagLast = 6, kKnobCount = 7;
 long long knob(int which);
 int set_knob(int which, long long value);
 // compute units of the current device (queried once per device)
@@ -97,6 +97,7 @@ struct GemmArgs {
   bf16_t* c2_list[kMaxBatch];
   int tiles_m, tiles_n;   // number of block tiles along each output dimension of one matrix
   int num_tiles;          // tiles actually computed, over the whole batch
+  int diag_last;          // 256x256 schedule, one symmetric matrix: its last `diag_last` diagonal tiles end the tile order
 };
 
 // the arguments of matrix b of a batch, as a single-matrix problem

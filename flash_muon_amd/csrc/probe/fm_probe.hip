@@ -4,8 +4,8 @@
 // ticks it took, so that the clock the chip holds under that load can be read off.  With operands
 // of zeros the chip stays at its full clock; with N(0,1)-like operands the power cap lowers the
 // clock, which is the ceiling that the GEMM kernels of this library work under on real data.
-#include "../../include/flashmuon.h"
-#include "fm_internal.h"
+// Not part of libflashmuon_hip.so: built into libflashmuon_probe.so, which only bench.py --mfma-probe loads.
+#include "../fm_internal.h"
 
 namespace fm {
 namespace {
@@ -49,12 +49,19 @@ __global__ __launch_bounds__(256) void mfma_peak_kernel(const uint4* __restrict_
 }  // namespace
 }  // namespace fm
 
-extern "C" int fm_probe_mfma_peak(const void* operands, int blocks, int iters, int launches, float* sink,
-                                  long long* clocks, fm_stream_t stream) {
-  if (!operands || !sink || !clocks) return FM_ERR_NULL;
-  if (blocks <= 0 || blocks > 1024 || iters <= 0 || launches <= 0) return FM_ERR_SHAPE;
+// `launches` launches of a kernel in which `blocks` workgroups of four waves each issue iters * 64
+// independent 32x32x16 bf16 MFMAs per wave on register operands taken from `operands` (blocks * 256 *
+// 128 bytes: zeros, or N(0,1) bf16 values).  After the last launch clocks[2*b] holds the shader cycles
+// and clocks[2*b + 1] the 100 MHz real-time ticks workgroup b spent in its loop; sink takes
+// blocks * 256 floats nobody needs.  The flop count is blocks * 4 * iters * 64 * 32768 per launch.
+// Returns 0, or 1 (a NULL pointer), 2 (a count out of range), 7 (launch failed).
+extern "C" __attribute__((visibility("default")))
+int fm_probe_mfma_peak(const void* operands, int blocks, int iters, int launches, float* sink,
+                       long long* clocks, void* stream) {
+  if (!operands || !sink || !clocks) return 1;
+  if (blocks <= 0 || blocks > 1024 || iters <= 0 || launches <= 0) return 2;
   for (int i = 0; i < launches; ++i)
     hipLaunchKernelGGL(fm::mfma_peak_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                        static_cast<const uint4*>(operands), sink, clocks, iters);
-  return hipGetLastError() == hipSuccess ? FM_OK : FM_ERR_LAUNCH;
+  return hipGetLastError() == hipSuccess ? 0 : 7;
 }

@@ -97,7 +97,12 @@ class Muon(torch.optim.Optimizer):
         ns_steps: The number of Newton-Schulz iteration steps to use.
         rank, world_size: required, as in the reference; only (0, 1) is implemented.
         batch: (not in the reference) how many same-shape matrices are orthogonalised per launch,
-            1..32; default 32.
+            1..32; default 32.  Memory: the Newton-Schulz scratch of a launch (four padded copies of
+            the iterate, two squares) is about 6.3 times the bytes of its bf16 matrices, 0.44 GB per
+            4096 x 11008 matrix and 14 GB for 32 of them (the reference holds about 0.3 GB, one
+            matrix at a time), taken from torch's caching allocator per call; a [batch, numel] bf16
+            staging buffer per group stays with the optimizer (2.9 GB at the default for that
+            shape).  A smaller batch shrinks both in proportion.
 
     Not for embeddings, the final fully connected layer or 0/1-D parameters; 4-D convolution
     filters are flattened over their last three dimensions.

@@ -15,8 +15,10 @@
  *     launch; asynchronous device faults surface at the caller's next synchronisation;
  *   - `ws`/`ws_bytes` is caller-provided scratch of at least the size the matching
  *     *_workspace_bytes() function returns (it may be NULL when that size is 0).
- *   - the library is stateless and re-entrant; two calls that share a workspace must be ordered
- *     on one stream.
+ *   - the entry points keep no state between calls and are re-entrant; two calls that share a
+ *     workspace must be ordered on one stream.  The exceptions are process-global: the tuning
+ *     knobs (fm_set_knob: one setting for all threads, to be changed only while no other thread is
+ *     inside a call) and the device array of fm_syrk_bf16_static.
  */
 #ifndef FLASHMUON_H
 #define FLASHMUON_H
@@ -56,7 +58,8 @@ FM_API const char* fm_version(void);
 
 /* Tuning knobs, for experiments and for tests that have to reach a particular schedule.  A
  * negative value gives the decision back to the library.  The environment variables
- * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS, FLASHMUON_NO_MID, FLASHMUON_NO_SUB64 and FLASHMUON_HALF set the initial
+ * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS, FLASHMUON_NO_MID, FLASHMUON_NO_SUB64, FLASHMUON_HALF
+ * and FLASHMUON_DIAG_LAST set the initial
  * values; they are read once, when the library is first used, never per call.  No counterpart in
  * the reference (its tuning is Triton's autotune table, flash_muon/matmul_transpose_triton.py:6-18).
  */
@@ -69,8 +72,11 @@ enum fm_knob {
                                   kernel) even where 64x64 sub-tiles over the whole k would do, and never run
                                   a whole product on such sub-tiles; 0: run every product of at most a
                                   sixteenth as many 256x256 tiles as workgroups on them (by estimate otherwise) */
-  FM_KNOB_HALF = 5             /* 1: always, 0: never run the 256x256 schedule on 128x256 half tiles (taken by
+  FM_KNOB_HALF = 5,            /* 1: always, 0: never run the 256x256 schedule on 128x256 half tiles (taken by
                                   itself when all of them fit into one round of workgroups) */
+  FM_KNOB_DIAG_LAST = 6        /* 0: the tiles left after the last full round of a symmetric product are the
+                                  last of the blocked tile order, whatever they are (otherwise: diagonal tiles,
+                                  which need one operand panel each and 10 of their 16 sub-tiles) */
 };
 FM_API int fm_set_knob(int knob, long long value);
 
@@ -108,9 +114,13 @@ FM_API size_t fm_syrk_workspace_bytes(int M, int K);
 
 /* fm_syrk_bf16 for callers that cannot allocate or hand over scratch memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
- * reference.  Same arguments and results as fm_syrk_bf16 minus ws / ws_bytes: the partial tiles go
- * to a 64 MiB array that the library holds in the device memory of every GPU it is used on, from the
- * first use until the process ends.  Nothing is allocated, freed or synchronised; the first call on
+ * reference.  Same arguments as fm_syrk_bf16 minus ws / ws_bytes, and the results of fm_syrk_bf16
+ * called with a workspace of 64 MiB: the partial tiles go to a 64 MiB array (256 slots of 256 KiB)
+ * that the library holds in the device memory of every GPU it is used on, from the first use until
+ * the process ends.  (Outputs of few tiles with a long k, which fm_syrk_bf16 cuts deeper along k when
+ * it is given the up to 192 MiB of fm_gemm_workspace_bytes, are cut as far as 256 slots allow; their
+ * fp32 sums then run in another order.  Sides that are not whole tiles run on the general schedule,
+ * without padded copies.)  Nothing is allocated, freed or synchronised; the first call on
  * a device looks the array's address up (do that once outside a graph capture).
  * Limits: M <= FM_STATIC_MAX_M and K <= FM_STATIC_MAX_K, otherwise FM_ERR_SHAPE.  All calls on one
  * GPU share the array, which keeps the last call's contents (nothing in it has to start at zero:
@@ -248,18 +258,6 @@ FM_API int fm_momentum_nesterov_batched(void* const* g, void* const* buf, int ba
                                  float w_buf, float w_nes, int nesterov, fm_stream_t stream);
 FM_API int fm_weight_update_batched(void* const* p, int p_dtype, const void* const* u_bf16, int batch,
                              int64_t n, float decay_mul, float alpha, fm_stream_t stream);
-
-/* ---------------------------------------------------------------------------------------------
- * Measurement aid, no counterpart in the reference: `launches` launches of a kernel in which
- * `blocks` workgroups of four waves each issue iters * 64 independent 32x32x16 bf16 MFMAs per wave on
- * register operands taken from `operands` (blocks * 256 * 128 bytes: zeros, or N(0,1) bf16 values).
- * After the last launch clocks[2*b] holds the shader cycles and clocks[2*b + 1] the 100 MHz
- * real-time ticks workgroup b spent in its loop; sink takes blocks * 256 floats nobody needs.
- * The flop count is blocks * 4 * iters * 64 * 32768 per launch.  bench.py --mfma-probe reports the
- * sustained rate and clock with it: the ceiling the power cap sets for MFMA work on real data.
- */
-FM_API int fm_probe_mfma_peak(const void* operands, int blocks, int iters, int launches, float* sink,
-                              long long* clocks, fm_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -192,6 +192,32 @@ def test_syrk_fast_last_round_in_space_or_along_k(lib, knobs, M, K, grid, no_sub
         assert float((got.float() - whole.float()).norm() / whole.float().norm()) < 1e-3
 
 
+@pytest.mark.parametrize("M,K,grid", [(8192, 128, -1), (2560, 256, 53), (4352, 64, 144), (3072, 192, 75), (3072, 64, 74)])
+def test_left_over_tiles_of_a_symmetric_product_are_diagonal_ones(lib, knobs, M, K, grid):
+    """The tiles left after the last full round of a symmetric product are taken from the end of the
+    diagonal (one operand panel each, 10 distinct sub-tiles of 16), the others close ranks in the blocked
+    order: 16 of 528 at 8192^2 (two whole 8x8 blocks of the order lose their diagonal), 2 of 55, 9 of 153,
+    3 and 4 of 78 (a block that loses part of its diagonal, or all of it).  Every tile must still be computed exactly
+    once: integer input against the exact product, and the same bits as the plain order (the DIAG_LAST
+    knob) on Gaussian input."""
+    knobs("FLASHMUON_GRID", grid)
+    X = _ints((M, K), M + K + 1)
+    want = _exact(X.double() @ X.double().T)
+    Xd = X.to(DEV)
+    Y = torch.full((M, M), float("nan"), dtype=torch.bfloat16, device=DEV)
+    st = lib.fm_syrk_bf16(Xd.data_ptr(), K, Y.data_ptr(), M, 1, M, K, None, 0, gpu_util._stream(Xd))
+    assert st == 0
+    assert torch.equal(Y.cpu(), want)
+    assert torch.equal(Y, Y.T)
+    g = torch.Generator().manual_seed(M + grid)
+    G = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    got = gpu_util.syrk(lib, G)
+    knobs("FLASHMUON_DIAG_LAST", 0)
+    plain = gpu_util.syrk(lib, G)
+    assert torch.equal(got, plain)
+    assert torch.equal(got, got.T)
+
+
 @pytest.mark.parametrize("no_sub64", [0, 1])
 def test_poly_and_axpby_fast_last_round_in_space(lib, knobs, no_sub64):
     """The epilogue operand, the fp32 diagonal and the per-row addition on the 64x64 sub-tiles."""

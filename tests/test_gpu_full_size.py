@@ -108,19 +108,23 @@ def _batched_ns(lib, Gs, steps=5):
     return outs
 
 
-@pytest.mark.parametrize("rows,cols,checked", [(4096, 4096, (0, 11)), (4096, 11008, (5, 15)), (11008, 4096, (2,))])
-def test_sixteen_per_launch_schedule(lib, rows, cols, checked):
-    """fm_newtonschulz_batched_bf16 with sixteen Llama-7B-sized matrices per launch, the schedule
-    Muon.step and bench.py run: the members in `checked` against the fp32 CPU oracle, every member
-    for finite values and against the single-matrix call (which differs only in which tiles are
-    summed from parts, i.e. in fp32 summation order)."""
-    n = 16
+@pytest.mark.parametrize("n,rows,cols,checked", [
+    (32, 4096, 4096, (0, 17, 31)), (32, 4096, 11008, (9, 31)), (32, 11008, 4096, (20,)),
+    (16, 4096, 4096, (0, 11)), (16, 4096, 11008, (5, 15)), (16, 11008, 4096, (2,))])
+def test_many_per_launch_schedules(lib, n, rows, cols, checked):
+    """fm_newtonschulz_batched_bf16 with n Llama-7B-sized matrices per launch.  Thirty-two is what
+    Muon.step and bench.py run on the Llama-7B set (flash_muon/muon.py:90-103 walks the same
+    parameters one by one): 32 x 136 and 32 x 688 tiles of 256x256 are whole rounds of 256
+    workgroups.  Sixteen end in a last round of tiles cut along k (2176 = 8 x 256 + 128 tiles), another
+    code path.  The members in `checked` against the fp32 CPU oracle, every member for finite values
+    and against the single-matrix call (which differs only in which tiles are summed from parts or run
+    on half tiles, i.e. in fp32 summation order)."""
     Gs = [synthetic.gradient_like_bf16(rows, cols, 8, 700 + i) for i in range(n)]
     dGs = [G.to(DEV) for G in Gs]
     outs = _batched_ns(lib, dGs)
     for i in checked:
         err = oracle.rel_fro(outs[i], oracle.newtonschulz(Gs[i], 5))
-        print("batch of 16, %dx%d, member %d: rel_fro %.3e" % (rows, cols, i, err), flush=True)
+        print("batch of %d, %dx%d, member %d: rel_fro %.3e" % (n, rows, cols, i, err), flush=True)
         assert err < 1e-2
     for i in range(n):
         assert bool(torch.isfinite(outs[i]).all())

@@ -188,3 +188,30 @@ def test_batched_step_matches_unbatched():
     for batch in (4, 32):
         for x, y, p0 in zip(res[1], res[batch], ps):
             assert oracle.rel_fro(x.double() - p0.double(), y.double() - p0.double()) < 4e-3
+
+
+def test_buckets_larger_than_a_launch_go_in_equal_chunks():
+    """A bucket of more same-shape parameters than one launch takes is handed over in chunks of equal
+    size (48 as 24 + 24, 70 as 24 + 24 + 22) at the default batch of 32: every parameter must move as
+    it does one matrix per launch (flash_muon/muon.py:90-103 walks them one by one), and no chunk may
+    be skipped or taken twice."""
+    shapes = [(384, 256)] * 48 + [(128, 512)] * 70
+    ps, gs = _make(shapes, 23)
+    ps = [p.float() for p in ps]
+    res = {}
+    for batch in (1, None):
+        params = _device_params(ps, gs)
+        opt = Muon(params, lr=LR, momentum=MU, rank=0, world_size=1, batch=batch)
+        opt.step()
+        torch.cuda.synchronize()
+        res[batch] = [q.data.cpu() for q in params]
+    for i, (x, y, p0) in enumerate(zip(res[1], res[None], ps)):
+        assert bool(torch.isfinite(y).all())
+        moved = y.double() - p0.double() * (1 - LR * WD)
+        assert float(moved.abs().max()) > 0, "parameter %d was not updated" % i
+        assert oracle.rel_fro(moved, x.double() - p0.double() * (1 - LR * WD)) < 6e-3, i
+    # two members against the oracle
+    for i in (30, 100):
+        ref_p, _, _, _ = oracle.muon_step([ps[i]], [gs[i]], [None], LR, WD, MU, True, 5)
+        assert oracle.rel_fro(res[None][i].double() - ps[i].double() * (1 - LR * WD),
+                              ref_p[0].double() - ps[i].double() * (1 - LR * WD)) < 1e-2
