@@ -79,7 +79,8 @@ def _interleaved(fns, calls, blocks, warm, torch):
 
 def _mfma_probe(torch):
     """Sustained rate and clock of MFMA-only work (fm_probe_mfma_peak), on zeros and on N(0,1) bf16
-    operands: about 150 ms of back-to-back launches each, the second half timed."""
+    operands, for the two MFMA shapes and with or without the GEMM's LDS fragment traffic: about
+    150 ms of back-to-back launches each, the second half timed."""
     import ctypes
     from flash_muon_amd import _lib, build
     if not os.path.exists(build.PROBE_LIB_PATH):
@@ -87,30 +88,36 @@ def _mfma_probe(torch):
     lib = ctypes.CDLL(build.PROBE_LIB_PATH)   # the probe is not part of the product library
     vp = ctypes.c_void_p
     lib.fm_probe_mfma_peak.restype = ctypes.c_int
-    lib.fm_probe_mfma_peak.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+    lib.fm_probe_mfma_peak.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp, ctypes.c_int, ctypes.c_int]
     blocks, iters, launches = 256, 256, 480
     sink = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
     clocks = torch.zeros(blocks * 2, dtype=torch.int64, device="cuda")
     g = torch.Generator(device="cuda").manual_seed(1)
     out = {}
-    for name, ops in (("zeros", torch.zeros(blocks * 256 * 64, dtype=torch.bfloat16, device="cuda")),
-                      ("gaussian", torch.randn(blocks * 256 * 64, generator=g, device="cuda").bfloat16())):
-        st = _lib.stream_ptr("cuda")
-        lib.fm_probe_mfma_peak(ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        lib.fm_probe_mfma_peak(ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st)
-        e0.record()
-        rc = lib.fm_probe_mfma_peak(ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st)
-        e1.record()
-        torch.cuda.synchronize()
-        assert rc == 0
-        ms = e0.elapsed_time(e1) / (launches // 2)
-        c = clocks.view(blocks, 2).double().mean(0)
-        flop = blocks * 4 * iters * 64 * 32768.0
-        out[name] = {"tflops": flop / ms / 1e9, "ms_per_launch": ms, "shader_cycles": float(c[0]),
+    data = (("zeros", torch.zeros(blocks * 256 * 64, dtype=torch.bfloat16, device="cuda")),
+            ("gaussian", torch.randn(blocks * 256 * 64, generator=g, device="cuda").bfloat16()))
+    for rep in range(2):   # every variant twice, in turn, so that drift of the box shows
+        for name, ops in data:
+            for shape, lds in ((0, 0), (1, 0), (0, 1), (1, 1)):
+                key = "%s_%s%s" % (name, ("32x32x16", "16x16x32")[shape], "_lds" if lds else "")
+                st = _lib.stream_ptr("cuda")
+                args = (ops.data_ptr(), blocks, iters, launches // 2, sink.data_ptr(), clocks.data_ptr(), st, shape, lds)
+                lib.fm_probe_mfma_peak(*args)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                lib.fm_probe_mfma_peak(*args)
+                e0.record()
+                rc = lib.fm_probe_mfma_peak(*args)
+                e1.record()
+                torch.cuda.synchronize()
+                assert rc == 0
+                ms = e0.elapsed_time(e1) / (launches // 2)
+                c = clocks.view(blocks, 2).double().mean(0)
+                flop = blocks * 4 * iters * 64 * 32768.0
+                out.setdefault(key, []).append(
+                    {"tflops": flop / ms / 1e9, "ms_per_launch": ms, "shader_cycles": float(c[0]),
                      "realtime_ticks_100mhz": float(c[1]), "clock_ghz": float(c[0] / c[1] / 10.0),
-                     "mfma_issue_fraction": iters * 64 * 32 / float(c[0])}
+                     "mfma_issue_fraction": iters * 64 * 32 / float(c[0])})
     return out
 
 
