@@ -149,6 +149,105 @@ __device__ __forceinline__ void stage(f32x16_t (&acc)[NR][4], Frag<NI>& f0, Frag
   tail_phase<F16, NI, ASLOT, BSLOT>(acc, f1, f0, smem, fa, voB, nB, ldsw);
 }
 
+// ---- whole tiles on 16x16x32 MFMAs --------------------------------------------------------------
+// A whole 256x256 tile runs on the 16x16x32 form of the instruction: on N(0,1) operands a loop of
+// nothing but MFMAs sustains 2.03 PFLOP/s with it and 1.78 with the 32x32x16 form, the power cap
+// allowing a clock of 2.0 against 1.77 GHz.  A wave's 128x128 block is 8 x 8 accumulator tiles of four
+// registers; a 64-wide k stage is two k32 substeps of 64 MFMAs and 16 fragment reads each.
+//
+// Layout.  A lane of a 16x16 accumulator tile holds four consecutive rows (4 (lane / 16) + r) of one
+// column (lane % 16) of the rows and columns its fragments were loaded with, and those are chosen so
+// that the write-out needs no exchange between lanes: LDS row l of an operand stage holds row
+// perm_a(l) of operand A's panel and row perm_b(l) of operand B's (permutations inside groups of 32
+// rows, applied where the copies fetch from global memory, so that a fragment is 16 consecutive LDS
+// rows).  Fragment i of A is then rows 32 (i / 2) + 8 g + 4 (i % 2) + r of the block for the lanes of
+// group g = lane / 16, and fragment j of B columns 32 (j / 2) + 2 n + j % 2 for lane n = lane % 16:
+// per 32x32 sub-block a lane holds 8 consecutive rows of 2 adjacent columns, i.e. after rounding a
+// 32-bit word of every one of 8 rows of C (two columns) and 16 bytes of two rows of C2 (eight rows).
+//
+// 16-byte chunk c of LDS row r sits at position c ^ swz16(r); the 16 rows of a fragment then cover
+// all 64 banks once per chunk column, and a fragment 16 rows further down is the same per-lane
+// address plus 2048 bytes: six address registers in all, the rest is immediate offsets.
+__device__ __forceinline__ int swz16(int row) { return (row >> 1) & 7; }
+__host__ __device__ constexpr int perm_a(int l) { return (l & ~31) + 8 * ((l >> 2) & 3) + 4 * ((l >> 4) & 1) + (l & 3); }
+__host__ __device__ constexpr int perm_b(int l) { return (l & ~31) + 2 * (l & 15) + ((l >> 4) & 1); }
+
+template <bool F16>
+__device__ __forceinline__ f32x4_t mfma_16x16x32(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+struct Frag16 { bf16x8_t a[8], b[8]; };
+// per-lane LDS byte addresses of fragment 0 for k32 substep kk: operand A in A slots 0 and 1
+// (a_lo, + OPER_BYTES) and in A slot 2 (a_hi), operand B in B slots 0 and 1
+struct FragAddr16 { uint32_t a_lo[2], a_hi[2], b[2]; };
+
+template <int ASLOT>
+__device__ __forceinline__ bf16x8_t read_a16(const unsigned char* smem, const FragAddr16& fa, int i, int kk) {
+  if constexpr (ASLOT == 2) return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_hi[kk] + i * 2048);
+  else return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_lo[kk] + ASLOT * OPER_BYTES + i * 2048);
+}
+template <int BSLOT>
+__device__ __forceinline__ bf16x8_t read_b16(const unsigned char* smem, const FragAddr16& fa, int j, int kk) {
+  return *reinterpret_cast<const bf16x8_t*>(smem + fa.b[kk] + BSLOT * OPER_BYTES + j * 2048);
+}
+
+// The 64 MFMAs of k32 substep KK of the stage in (ASLOT, BSLOT).  The 16 fragment reads of the
+// next substep (the second half of this stage, or the first half of the next one) ride on the first 32
+// of them, in the order the next substep needs them.  During substep 0 the 8 copies of operand A of
+// the stage two ahead go out, into the A slot the previous stage has left; during the first half of
+// substep 1, behind the barrier of the stage, the 8 copies of operand B of that stage, into the B
+// slot this stage has just read for the last time.
+template <bool F16, int ASLOT, int BSLOT, int KK, bool FIRST>
+__device__ __forceinline__ void substep16(f32x4_t (&acc)[8][8], const Frag16& cur, Frag16& nxt,
+                                          const unsigned char* smem, const FragAddr16& fa,
+                                          const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                          const bf16_t* gA, const bf16_t* gB, uint32_t ldsw) {
+  constexpr int AFREE = (ASLOT + 2) % 3, ANEXT = (ASLOT + 1) % 3, BNEXT = BSLOT ^ 1;
+#pragma unroll
+  for (int q = 0; q < 64; ++q) {
+    if ((q & 1) == 0 && q < 32) {
+      const int t = q >> 1;   // read t of the next substep: a0, b0 .. b7, a1 .. a7
+      if constexpr (KK == 0) {
+        if (t == 0) nxt.a[0] = read_a16<ASLOT>(smem, fa, 0, 1);
+        else if (t <= 8) nxt.b[t - 1] = read_b16<BSLOT>(smem, fa, t - 1, 1);
+        else nxt.a[t - 8] = read_a16<ASLOT>(smem, fa, t - 8, 1);
+      } else {
+        if (t == 0) nxt.a[0] = read_a16<ANEXT>(smem, fa, 0, 0);
+        else if (t <= 8) nxt.b[t - 1] = read_b16<BNEXT>(smem, fa, t - 1, 0);
+        else nxt.a[t - 8] = read_a16<ANEXT>(smem, fa, t - 8, 0);
+      }
+    }
+    if constexpr (KK == 0) {
+      if ((q & 7) == 5) dma16o(voA[q >> 3], gA, ldsw, a_slot_off(AFREE) + (q >> 3) * 4096);
+    } else {
+      if ((q & 3) == 1 && q < 32) dma16o(voB[q >> 2], gB, ldsw, b_slot_off(BSLOT) + (q >> 2) * 4096);
+    }
+    if constexpr (FIRST && KK == 0) {
+      const f32x4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+      acc[q >> 3][q & 7] = mfma_16x16x32<F16>(cur.a[q >> 3], cur.b[q & 7], zero);
+    } else {
+      acc[q >> 3][q & 7] = mfma_16x16x32<F16>(cur.a[q >> 3], cur.b[q & 7], acc[q >> 3][q & 7]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// One k stage.  At the barrier between its substeps every wave has waited for its copies of the
+// next stage (all but the 8 newest, operand A of the stage after), and every fragment read of this
+// stage has returned, so that its B slot may be refilled.
+template <bool F16, int ASLOT, int BSLOT, bool FIRST = false>
+__device__ __forceinline__ void stage16(f32x4_t (&acc)[8][8], Frag16& f0, Frag16& f1, const unsigned char* smem,
+                                        const FragAddr16& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                        const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
+  substep16<F16, ASLOT, BSLOT, 0, FIRST>(acc, f0, f1, smem, fa, voA, voB, nA, nB, ldsw);
+  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  substep16<F16, ASLOT, BSLOT, 1, false>(acc, f1, f0, smem, fa, voA, voB, nA, nB, ldsw);
+}
+
 // ---- a diagonal tile of a symmetric product as one item of the half-tile schedule ---------------
 // Of the 8 x 8 MFMA tiles of a diagonal 256x256 tile only those on or below the diagonal are
 // distinct: 36, against the 32 of a half tile, 9 per wave.  Waves 0 and 1 take the lower triangles
@@ -713,6 +812,173 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
 #undef FM_ET
 }
 
+// ---- write-out of a whole tile from the 16x16 accumulator tiles ---------------------------------
+// The wave's block is 128 rows x 128 columns at (row0, col0); per 32x32 sub-block (I, J) a lane (n =
+// lane % 16, g = lane / 16) holds rows 32 I + 8 g + 4 a + r of columns 32 J + 2 n + b in register r of
+// tile (2 I + a, 2 J + b).  Rounded pairs (b = 0, 1) are 32-bit words of a row of C: they are staged
+// row-major, a quarter (32 rows x 128 columns) at a time, and read back 16 bytes per lane.  Rounded
+// pairs of rows are collected column by column over two quarters (64 rows = 128 bytes per column of
+// the block) and leave as whole cache lines of C2, 8 lanes per row of it.  The operand E is read
+// transposed (ET), 8 consecutive rows of one column per lane and load, which is exactly what the lane
+// holds of that column, so the arithmetic happens in registers.  Both copies carry the same bits.
+// MODE, diag, dshift: as for epilogue_regs (MFMA tile there = 32x32 sub-block here).
+constexpr int QD_PITCH = 256;   // staged row of the direct copy: 128 values; 64-byte groups XOR-swizzled by row / 8
+static_assert(32 * QD_PITCH <= QT_BYTES, "the direct staging of the 16x16 write-out fits the region of the other one");
+
+template <bool F16, int MODE>
+__device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, int dshift, const f32x4_t (&acc)[8][8],
+                                                unsigned char* T, int row0, int col0, int lane) {
+  // derived from `lane` anew for every tile (see epilogue_regs)
+  asm volatile("" : "+v"(lane));
+  constexpr bool has_e = !F16 && MODE != 0;
+  const int n = lane & 15, grp = lane >> 4;
+  const bool direct = g.C != nullptr;
+  const bool mirror = g.C2 != nullptr && !diag;
+  const bool dout = diag && g.diag_out != nullptr;
+  const float alpha = g.alpha, beta = g.beta;
+  float* const RA = reinterpret_cast<float*>(T + QT_BYTES);
+  // direct staging: this lane writes rows 8 grp + 4 a + r, the 4 bytes of columns 32 J + 2 n .. + 1, at
+  // 64-byte group J ^ grp of the row; it reads row 4 it + lane / 16, columns 8 (lane % 16) .. + 7
+  unsigned char* const tw = T + (8 * grp) * QD_PITCH + 4 * n;
+  const unsigned char* const tr = T + (lane >> 4) * QD_PITCH + (lane & 3) * 16;
+  const int rgrp = (lane >> 2) & 3;   // 64-byte group of what it reads, before the swizzle
+  // mirrored staging: rows 32 (I % 2) + 8 grp + 4 a .. + 3 of column 32 J + 2 n + b; read as in epilogue_regs
+  unsigned char* const mw = T + QM_OFFSET + (2 * n) * QM_PITCH + 16 * grp;
+  const unsigned char* const mr = T + QM_OFFSET + (lane >> 3) * QM_PITCH + (lane & 7) * 16;
+  const uint32_t et_lane = (uint32_t)((2 * n) * (int)g.ldet + 8 * grp) * 2u;
+  const uint32_t c2_lane = (uint32_t)((lane >> 3) * (int)g.c2_rs + (lane & 7) * 8) * 2u;
+  const uint32_t c_lane = (uint32_t)((lane >> 4) * (int)g.c_rs + (lane & 15) * 8) * 2u;
+  const __amdgpu_buffer_rsrc_t et_buf = block_rsrc(g.ET + (int64_t)col0 * g.ldet + row0);
+  const __amdgpu_buffer_rsrc_t c2_buf = block_rsrc(g.C2 + (int64_t)col0 * g.c2_rs + row0);
+  const __amdgpu_buffer_rsrc_t c_buf = block_rsrc(g.C + (int64_t)row0 * g.c_rs + col0);
+  const int et_col = 2 * (int)g.ldet, c2_col = 16 * (int)g.c2_rs, c_row = 8 * (int)g.c_rs;   // bytes: 1 column, 8 columns, 4 rows
+#define FM_ET16(I, J, b) buf_load16(et_buf, et_lane, (32 * (J) + (b)) * et_col + 64 * (I))
+
+  uint4 ev[4][2];
+  if constexpr (has_e) {
+    // the block's 128 additions to alpha (zeros when there are none), before any store of this tile
+    float2 ra = {0.0f, 0.0f};
+    if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+    *reinterpret_cast<float2*>(RA + lane * 2) = ra;
+#pragma unroll
+    for (int J = 0; J < 4; ++J)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) ev[J][b] = FM_ET16(0, J, b);
+  }
+
+#pragma unroll
+  for (int I = 0; I < 4; ++I) {
+    f32x4_t al[2];
+    if constexpr (has_e) {
+#pragma unroll
+      for (int a = 0; a < 2; ++a) {
+        al[a] = *reinterpret_cast<const f32x4_t*>(RA + 32 * I + 8 * grp + 4 * a);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) al[a][e] += alpha;
+      }
+    }
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+      // one sub-block at a time (see epilogue_regs)
+      __builtin_amdgcn_sched_barrier(0);
+      auto block = [&](auto dout_tag) {
+        constexpr bool DOUT = decltype(dout_tag)::value;
+        float v[2][2][4];   // [a][b][r]
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[a][b][r] = acc[2 * I + a][2 * J + b][r];
+        if constexpr (has_e) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const uint32_t w[4] = {ev[J][b].x, ev[J][b].y, ev[J][b].z, ev[J][b].w};   // rows 2 k, 2 k + 1 of the lane's eight
+            if (I < 3) ev[J][b] = FM_ET16(I + 1, J, b);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const uint32_t ww = w[2 * a + (r >> 1)];
+                const float ef = elem_to_f32<F16>((unsigned short)((r & 1) ? (ww >> 16) : (ww & 0xffffu)));
+                const float x = MODE == 2 ? beta * v[a][b][r] : v[a][b][r];
+                v[a][b][r] = __builtin_fmaf(al[a][r], ef, x);
+              }
+          }
+        }
+        if constexpr (DOUT) {
+          // row 8 grp + 4 a + r meets column 2 n + b: the lanes with n / 4 == grp hold two elements of the
+          // diagonal, rows 2 n and 2 n + 1 of the sub-block; they are split off in fp32 and stored as zero
+          float dv[2] = {0.0f, 0.0f};
+#pragma unroll
+          for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const bool on = 2 * n + b == 8 * grp + 4 * a + r;
+                dv[b] = on ? v[a][b][r] : dv[b];
+                v[a][b][r] = on ? 0.0f : v[a][b][r];
+              }
+          if ((n >> 2) == grp) {
+            g.diag_out[row0 + 32 * I + 2 * n] = dv[0];
+            g.diag_out[row0 + 32 * I + 2 * n + 1] = dv[1];
+          }
+        }
+        if (direct) {
+#pragma unroll
+          for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              *reinterpret_cast<uint32_t*>(tw + (4 * a + r) * QD_PITCH + 64 * (J ^ grp)) = pack2<F16>(v[a][0][r], v[a][1][r]);
+        }
+        if (mirror) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+              *reinterpret_cast<uint2*>(mw + (32 * J + b) * QM_PITCH + 64 * (I & 1) + 8 * a) =
+                  uint2{pack2<F16>(v[a][b][0], v[a][b][1]), pack2<F16>(v[a][b][2], v[a][b][3])};
+        }
+      };
+      if (dout && J == I + dshift) block(std::true_type{});
+      else block(std::false_type{});
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (has_e) {
+      if (I == 3) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): see epilogue_regs
+    }
+    if (direct) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        uint4 d[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it)   // rows 4 (4 half + it) + lane / 16: their 64-byte groups are swizzled by 2 half + it / 2
+          d[it] = *reinterpret_cast<const uint4*>(tr + 4 * (4 * half + it) * QD_PITCH + 64 * (rgrp ^ (2 * half + (it >> 1))));
+#pragma unroll
+        for (int it = 0; it < 4; ++it) buf_store16(c_buf, c_lane, (8 * I + 4 * half + it) * c_row, d[it]);
+      }
+    }
+    if (mirror && (I & 1)) {   // two quarters of the mirrored copy: 128 columns x 128 bytes
+#pragma unroll
+      for (int cg = 0; cg < 4; ++cg) {
+        uint2 d[4][2];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const unsigned char* src = mr + 8 * (4 * cg + it) * QM_PITCH;
+          d[it][0] = *reinterpret_cast<const uint2*>(src);
+          d[it][1] = *reinterpret_cast<const uint2*>(src + 8);
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+          buf_store16(c2_buf, c2_lane, (4 * cg + it) * c2_col + 128 * (I >> 1),
+                      uint4{d[it][0].x, d[it][0].y, d[it][1].x, d[it][1].y});
+      }
+    }
+  }
+#undef FM_ET16
+}
+
 // The schedule works on items: item i is base part i % ksplit of tile i / ksplit, where every tile's
 // k range is cut into `ksplit` equal base parts (1 unless there are too few tiles to fill the chip
 // and k is long).  Items [0, rounds * grid) run one per workgroup in `rounds` full rounds; the `rem`
@@ -1079,6 +1345,109 @@ __device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, in
   }
 }
 
+// accumulators of the 32-row group I of a wave's 128x128 block (16x16 tiles) -> F, as stage_store
+template <int I>
+__device__ __forceinline__ void stage_store16(const f32x4_t (&acc)[8][8], float* F, int lane) {
+  const int n = lane & 15, grp = lane >> 4;
+#pragma unroll
+  for (int J = 0; J < 4; ++J)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int col = 32 * J + 2 * n + b;
+      float* const dst = F + col * QF_PITCH;
+      const int x = ((col >> 3) & 7) << 2;
+#pragma unroll
+      for (int a = 0; a < 2; ++a) *reinterpret_cast<f32x4_t*>(dst + ((8 * grp + 4 * a) ^ x)) = acc[2 * I + a][2 * J + b];
+    }
+}
+
+// A whole 256x256 tile (or a part of one along k): n k stages from (gA, gB) on through the operand
+// ring on 16x16x32 MFMAs, then the write-out, or the hand-over of the fp32 sums to `slot`.
+template <bool F16, int MODE>
+__device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n, float* slot, unsigned char* smem,
+                                             const FragAddr16& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                             const bf16_t* gA, const bf16_t* gB, uint32_t ldsw, int row0, int col0,
+                                             int lane, int wave) {
+  f32x4_t acc[8][8];   // started from zero by the first substep of the first stage
+  {
+    Frag16 f0, f1;
+    // stages past the end are the last stage again (into slots nobody reads), so that the number
+    // of copies in flight is the same at every wait
+    const int last = n - 1;
+    const int k1 = last < 1 ? last : 1;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, b_slot_off(0) + q * 4096);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, b_slot_off(1) + q * 4096);
+    wait_vmcnt<16>();
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 8; ++q) f0.a[q] = read_a16<0>(smem, fa, q, 0);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) f0.b[q] = read_b16<0>(smem, fa, q, 0);
+    // the slots come round every 6 stages; the first stage stands apart
+#define FM_STAGE_T(AS, BS, S, FIRST)                                                             \
+    {                                                                                            \
+      const int kn = (S) + 2 < last ? (S) + 2 : last;                                            \
+      stage16<F16, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
+    }
+#define FM_STAGE(AS, BS, S) FM_STAGE_T(AS, BS, S, false)
+    FM_STAGE_T(0, 0, 0, true)
+    int s = 1;
+    for (; s + 6 <= n; s += 6) {
+      FM_STAGE(1, 1, s)
+      FM_STAGE(2, 0, s + 1)
+      FM_STAGE(0, 1, s + 2)
+      FM_STAGE(1, 0, s + 3)
+      FM_STAGE(2, 1, s + 4)
+      FM_STAGE(0, 0, s + 5)
+    }
+    if (s < n) {
+      FM_STAGE(1, 1, s)
+      if (s + 1 < n) {
+        FM_STAGE(2, 0, s + 1)
+        if (s + 2 < n) {
+          FM_STAGE(0, 1, s + 2)
+          if (s + 3 < n) {
+            FM_STAGE(1, 0, s + 3)
+            if (s + 4 < n) FM_STAGE(2, 1, s + 4)
+          }
+        }
+      }
+    }
+#undef FM_STAGE_T
+#undef FM_STAGE
+    wait_vmcnt<0>();
+    __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
+  }
+  unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
+  if (slot) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
+    const EpiLds L = epi_lds(wave_lds);
+    int sl = lane;   // per-lane offsets derived anew for every tile, not kept across the main loop
+    asm volatile("" : "+v"(sl));
+#define FM_QUARTER(q)                                                        \
+    stage_store16<q>(acc, L.F, sl);                                            \
+    copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, sl);
+    FM_QUARTER(0)
+    FM_QUARTER(1)
+    FM_QUARTER(2)
+    FM_QUARTER(3)
+#undef FM_QUARTER
+  } else {
+    // (the accumulators are pinned to their registers first, on this branch only: see the note on
+    // element reads at epilogue_regs)
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+    epilogue_regs16<F16, MODE>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane);
+  }
+}
+
 // MODE: how whole tiles are written out (see epilogue_regs); chosen by the host from E and beta
 template <bool F16, int MODE, int NI>
 __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
@@ -1100,10 +1469,21 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
 
   const uint32_t ldsw = FM_LDS_ADDR(smem) + wave * 1024;   // where this wave's copies land inside a slot
 
+  // whole tiles (NI == 4) run on 16x16x32 MFMAs: row = lane % 16 of a fragment's 16 LDS rows, k quarter = lane / 16
+  FragAddr16 fa16;
+  if constexpr (NI == 4) {
+    const int ra = wm * 128 + (lane & 15), rb = wn * 128 + (lane & 15);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      fa16.a_lo[kk] = (uint32_t)(ra * ROWB + (((4 * kk + (lane >> 4)) ^ swz16(ra)) << 4));
+      fa16.a_hi[kk] = fa16.a_lo[kk] + a_slot_off(2);
+      fa16.b[kk] = (uint32_t)(rb * ROWB + (((4 * kk + (lane >> 4)) ^ swz16(rb)) << 4)) + b_slot_off(0);
+    }
+  }
   // per-lane fragment addresses (row = lane % 32 of the fragment's 32 rows, k half = lane / 32)
   FragAddr<NI> fa;
 #pragma unroll
-  for (int i = 0; i < NI; ++i) {
+  for (int i = 0; i < (NI == 4 ? 0 : NI); ++i) {
     const int ra = wm * (32 * NI) + i * 32 + (lane & 31);
     const uint32_t ao = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
 #pragma unroll
@@ -1113,7 +1493,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     }
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < (NI == 4 ? 0 : 4); ++i) {
     const int rb = wn * 128 + i * 32 + (lane & 31);
     const uint32_t bo = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
 #pragma unroll
@@ -1160,9 +1540,15 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int row = (q * 4 + wave) * 8 + (lane >> 3);
-      const int chunk = (lane & 7) ^ swz(row);
-      if (q < 2 * NI) voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
-      voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
+      if constexpr (NI == 4) {   // LDS row `row` holds row perm_a(row) of A's panel and perm_b(row) of B's
+        const int chunk = (lane & 7) ^ swz16(row);
+        voA[q] = (uint32_t)(perm_a(row) * (int)g.lda + chunk * 8) * 2u;
+        voB[q] = (uint32_t)(perm_b(row) * (int)g.ldb + chunk * 8) * 2u;
+      } else {
+        const int chunk = (lane & 7) ^ swz(row);
+        if (q < 2 * NI) voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
+        voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
+      }
     }
     const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
     const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
@@ -1174,6 +1560,13 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
         continue;
       }
     }
+
+    if constexpr (NI == 4) {   // whole tiles, or parts of them along k
+      const bool diag = g.symmetric && ti == tj;
+      float* const slot = n != p.nk ? p.partials + (size_t)slot_id * PART_FLOATS : nullptr;
+      whole_tile16<F16, MODE>(g, diag, n, slot, smem, fa16, voA, voB, gA, gB, ldsw, m0 + wm * 128, n0 + wn * 128, lane, wave);
+      __syncthreads();   // the next tile's copies land in the memory the staging just used
+    } else {   // 128x256 half tiles: 32x32x16 MFMAs
 
     f32x16_t acc[NI][4];   // started from zero by the first substep of the first stage
 
@@ -1246,26 +1639,12 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
         _Pragma("unroll") for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));        \
       epilogue_regs<F16, MODE, NI, 0>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane); \
     }
-    if constexpr (NI == 4) {
-      if (split) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
-        const EpiLds L = epi_lds(wave_lds);
-        float* const slot = p.partials + (size_t)slot_id * PART_FLOATS;
-#define FM_QUARTER(q)                                                        \
-        stage_store<q, 4>(acc, L.F, lane);                                     \
-        copy_stage_to_ws(L.F, slot + (wave * 4 + q) * QUARTER_FLOATS, lane);
-        FM_QUARTER(0)
-        FM_QUARTER(1)
-        FM_QUARTER(2)
-        FM_QUARTER(3)
-#undef FM_QUARTER
-      } else {
-        FM_WRITE_OUT
-      }
-    } else {
-      FM_WRITE_OUT
-    }
+    (void)split;
+    (void)slot_id;
+    FM_WRITE_OUT
 #undef FM_WRITE_OUT
     __syncthreads();   // the next tile's copies land in the memory the staging just used
+    }   // NI != 4
   }
 }
 
