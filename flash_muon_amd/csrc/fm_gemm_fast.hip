@@ -1207,10 +1207,13 @@ __device__ __forceinline__ void diag_item(const GemmArgs& g, int m0, int n, unsi
 }
 
 // ---- 64x64 sub-tiles of the tiles left over after the last full round ---------------------------
-// One workgroup per sub-tile, four waves of 32x32 (one MFMA tile each), the whole k range, so the
-// result needs no second pass and is summed in the same k order as a whole tile.  A sub-tile moves
-// four times the operand bytes per flop of a 256x256 tile and is bound by the copy path (16 KiB per
-// stage against 4 MFMAs per wave), hence a deep ring: 8 stages of 16 KiB, 7 in flight.
+// One workgroup per sub-tile, four waves of 32x32 (2 x 2 accumulator tiles of the 16x16x32 MFMA), the
+// whole k range, so the result needs no second pass and is summed in the same k order as a whole tile.
+// A sub-tile moves four times the operand bytes per flop of a 256x256 tile and is bound by the copy
+// path (16 KiB per stage against 8 MFMAs per wave), hence a deep ring: 8 stages of 16 KiB, 7 in
+// flight.  The fragment reads of a stage are issued a stage ahead, behind the barrier that says it
+// has landed everywhere, and ride on the MFMAs of the stage before: wait, barrier, reads and MFMAs one
+// after the other cost 510 cycles a stage where the MFMAs take 128.
 constexpr int SUB = 64;
 constexpr int SUB_OPER = SUB * ROWB;          // 64 rows of one operand stage: 8 KiB
 constexpr int SUB_STAGE = 2 * SUB_OPER;
@@ -1244,37 +1247,69 @@ __device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, in
 #pragma unroll
     for (int q = 0; q < 2; ++q) dma16(voB[q], gB + stage * BKF, base + SUB_OPER + q * 1024);
   };
-  uint32_t ao, bo;
-  {
-    const int ra = wm * 32 + (lane & 31), rb = wn * 32 + (lane & 31);
-    ao = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
-    bo = (uint32_t)(SUB_OPER + rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
-  }
-
-  f32x16_t acc;
+  // per-lane fragment addresses inside a stage: [fragment of 16 rows][k32 substep]
+  uint32_t ao[2][2], bo[2][2];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+  for (int i = 0; i < 2; ++i) {
+    const int ra = wm * 32 + 16 * i + (lane & 15), rb = wn * 32 + 16 * i + (lane & 15);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      ao[i][kk] = (uint32_t)(ra * ROWB + (((4 * kk + (lane >> 4)) ^ swz(ra)) << 4));
+      bo[i][kk] = (uint32_t)(SUB_OPER + rb * ROWB + (((4 * kk + (lane >> 4)) ^ swz(rb)) << 4));
+    }
+  }
+  struct SubFrag { bf16x8_t a[2][2], b[2][2]; };   // [fragment][substep]
+  auto read_frag = [&](SubFrag& f, const unsigned char* st, int t) {   // read t of a stage's eight: substep t / 4, a0 b0 a1 b1
+    const int kk = t >> 2, i = (t >> 1) & 1;
+    if (t & 1) f.b[i][kk] = *reinterpret_cast<const bf16x8_t*>(st + bo[i][kk]);
+    else f.a[i][kk] = *reinterpret_cast<const bf16x8_t*>(st + ao[i][kk]);
+  };
+
+  f32x4_t acc[2][2];
   // stages past the end are the last stage again (into slots nobody reads), so that the number of
   // copies in flight is the same at every wait
 #pragma unroll
   for (int s = 0; s < SUB_DEPTH - 1; ++s) issue(s < nk ? s : nk - 1, s);
-  for (int s = 0; s < nk; ++s) {
-    wait_vmcnt<4 * (SUB_DEPTH - 2)>();   // my copies of stage s have landed ...
-    __syncthreads();                     // ... and everybody's; stage s-1 is read out everywhere
-    {
-      const int nx = s + SUB_DEPTH - 1;
-      issue(nx < nk ? nx : nk - 1, nx & (SUB_DEPTH - 1));
-    }
-    const unsigned char* st = smem + (s & (SUB_DEPTH - 1)) * SUB_STAGE;
-    bf16x8_t fa[4], fb[4];
+  wait_vmcnt<4 * (SUB_DEPTH - 2)>();   // stage 0 has landed
+  __syncthreads();
+  SubFrag f0, f1;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      fa[ks] = *reinterpret_cast<const bf16x8_t*>(st + (ao ^ (ks << 5)));
-      fb[ks] = *reinterpret_cast<const bf16x8_t*>(st + (bo ^ (ks << 5)));
-    }
+  for (int t = 0; t < 8; ++t) read_frag(f0, smem, t);
+  // One iteration: my copies of stage s + 1 have landed, and behind the barrier everybody's, while
+  // nobody reads stage s - 1 any more (its fragments were multiplied before the barrier), so its slot
+  // takes the copies of stage s + 7; the fragments of stage s + 1 are asked for while those of stage
+  // s, read an iteration ago, are multiplied.  (A bare barrier: the reads asked for an iteration ago
+  // may still be on their way, their slot is not refilled before they have been multiplied;
+  // __syncthreads() would wait for them here.)
+  auto iter = [&](int s, const SubFrag& cur, SubFrag& nxt, auto first_tag) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" :: "n"(4 * (SUB_DEPTH - 3)) : "memory");
+    const int nx = s + SUB_DEPTH - 1;
+    const int nstage = nx < nk ? nx : nk - 1;
+    const uint32_t nbase = ldsw + (nx & (SUB_DEPTH - 1)) * SUB_STAGE;
+    const unsigned char* st = smem + ((s + 1) & (SUB_DEPTH - 1)) * SUB_STAGE;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) acc = mfma_32x32x16<F16>(fa[ks], fb[ks], acc);
+    for (int q = 0; q < 8; ++q) {   // MFMA q: substep q / 4, tile (q / 2 % 2, q % 2)
+      if (q < 2) dma16(voA[q], gA + nstage * BKF, nbase + q * 1024);
+      else if (q < 4) dma16(voB[q - 2], gB + nstage * BKF, nbase + SUB_OPER + (q - 2) * 1024);
+      read_frag(nxt, st, q);
+      const int kk = q >> 2, i = (q >> 1) & 1, j = q & 1;
+      if constexpr (FIRST) {
+        if (kk == 0) acc[i][j] = mfma_16x16x32<F16>(cur.a[i][kk], cur.b[j][kk], f32x4_t{0.0f, 0.0f, 0.0f, 0.0f});
+        else acc[i][j] = mfma_16x16x32<F16>(cur.a[i][kk], cur.b[j][kk], acc[i][j]);
+      } else {
+        acc[i][j] = mfma_16x16x32<F16>(cur.a[i][kk], cur.b[j][kk], acc[i][j]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  iter(0, f0, f1, std::true_type{});
+  int s = 1;
+  for (; s + 2 <= nk; s += 2) {
+    iter(s, f1, f0, std::false_type{});
+    iter(s + 1, f0, f1, std::false_type{});
   }
+  if (s < nk) iter(s, f1, f0, std::false_type{});
   wait_vmcnt<0>();
   __syncthreads();   // no copy in flight and no wave still reading: the ring is free
 
@@ -1282,13 +1317,12 @@ __device__ __forceinline__ void sub64_tile(const GemmArgs& g, int ti, int tj, in
   // the direct pass writes 1 row x 16 columns per lane and puts the rounded values back, the
   // transposed pass 16 rows x 1 column per lane, so both copies carry the same bits
   float* const F = reinterpret_cast<float*>(smem + wave * (32 * SUB_F_PITCH * 4));
-  {
-    const int c = lane & 31, rg = 4 * (lane >> 5);
+  {   // register r of tile (i, j) of lane l is row 16 i + 4 (l / 16) + r, column 16 j + l % 16 of the block
+    const int c = lane & 15, rg = 4 * (lane >> 4);
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const f32x4_t v = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
-      *reinterpret_cast<f32x4_t*>(F + c * SUB_F_PITCH + 8 * q + rg) = v;
-    }
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) *reinterpret_cast<f32x4_t*>(F + (16 * j + c) * SUB_F_PITCH + 16 * i + rg) = acc[i][j];
   }
   const int row0 = m0 + wm * 32, col0 = n0 + wn * 32;
   // a block of a diagonal sub-tile holds its own mirror image (or is one of a pair of blocks that
