@@ -84,6 +84,17 @@ __device__ __forceinline__ void dma16o(uint32_t voff, const void* sbase, uint32_
                :: "v"(voff), "s"(sbase), "s"(lds_base), "n"(off) : "memory", "scc", "m0");
 }
 
+// The same copy in two statements with other instructions between them: the destination goes to M0
+// first (the instruction between is the wait state the copy needs after a write of M0), the copy
+// itself follows.  Nothing between the two may write M0; tests/test_generated_code.py looks for that
+// in the generated code.
+__device__ __forceinline__ void dma16_m0(uint32_t lds_base, int off) {
+  asm volatile("s_add_i32 m0, %0, %1" :: "s"(lds_base), "n"(off) : "scc", "m0");
+}
+__device__ __forceinline__ void dma16_go(uint32_t voff, const void* sbase) {
+  asm volatile("global_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase) : "memory");
+}
+
 // The 4 NI MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The NI + 4 fragment reads of
 // the next substep ride on the first ones, and copies Q0 .. Q1-1 of operand A of the stage two
 // ahead (into the A slot that the previous stage has left) go out between the others, so that the
@@ -207,6 +218,10 @@ __device__ __forceinline__ void substep16(f32x4_t (&acc)[8][8], const Frag16& cu
                                           const uint32_t (&voA)[8], const uint32_t (&voB)[8],
                                           const bf16_t* gA, const bf16_t* gB, uint32_t ldsw) {
   constexpr int AFREE = (ASLOT + 2) % 3, ANEXT = (ASLOT + 1) % 3, BNEXT = BSLOT ^ 1;
+  // every fragment of this substep was asked for half a substep ago: one wait for all of them, said
+  // in the form the compiler's bookkeeping of outstanding reads understands, instead of one in front
+  // of the first use of each
+  if constexpr (KK == 0) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
 #pragma unroll
   for (int q = 0; q < 64; ++q) {
     if ((q & 1) == 0 && q < 32) {
@@ -221,10 +236,13 @@ __device__ __forceinline__ void substep16(f32x4_t (&acc)[8][8], const Frag16& cu
         else nxt.a[t - 8] = read_a16<ANEXT>(smem, fa, t - 8, 0);
       }
     }
+    // (a copy is two statements, M0 and the copy, one MFMA apart, in the slots that carry no read)
     if constexpr (KK == 0) {
-      if ((q & 7) == 5) dma16o(voA[q >> 3], gA, ldsw, a_slot_off(AFREE) + (q >> 3) * 4096);
+      if ((q & 7) == 5) dma16_m0(ldsw, a_slot_off(AFREE) + (q >> 3) * 4096);
+      if ((q & 7) == 7) dma16_go(voA[q >> 3], gA);
     } else {
-      if ((q & 3) == 1 && q < 32) dma16o(voB[q >> 2], gB, ldsw, b_slot_off(BSLOT) + (q >> 2) * 4096);
+      if ((q & 3) == 1 && q < 32) dma16_m0(ldsw, b_slot_off(BSLOT) + (q >> 2) * 4096);
+      if ((q & 3) == 3 && q < 32) dma16_go(voB[q >> 2], gB);
     }
     if constexpr (FIRST && KK == 0) {
       const f32x4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -244,7 +262,8 @@ __device__ __forceinline__ void stage16(f32x4_t (&acc)[8][8], Frag16& f0, Frag16
                                         const FragAddr16& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
                                         const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
   substep16<F16, ASLOT, BSLOT, 0, FIRST>(acc, f0, f1, smem, fa, voA, voB, nA, nB, ldsw);
-  asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
+  asm volatile("s_barrier" ::: "memory");
   substep16<F16, ASLOT, BSLOT, 1, false>(acc, f1, f0, smem, fa, voA, voB, nA, nB, ldsw);
 }
 

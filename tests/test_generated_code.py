@@ -109,3 +109,49 @@ def test_gemm_kernels_do_not_spill(assembly):
     gemm = {k: v for k, v in sizes.items() if "gemm_nt" in k}
     assert len(gemm) >= 6, sorted(sizes)           # rounds x 4 instances, reduce x 2, mid x 2
     assert all(v == 0 for v in gemm.values()), {k: v for k, v in gemm.items() if v}
+
+
+def test_every_copy_finds_the_m0_its_statement_or_the_one_before_it_set(assembly):
+    """A copy into LDS takes its destination from M0.  Most statements set M0 and copy in one; the
+    main loop of the whole tiles sets M0 in one statement and copies in a later one, with MFMAs and
+    LDS reads between them.  In the code as built every copy must follow a write of M0 from an
+    assembly statement with nothing between them that writes M0 or leaves the straight line (a label, a
+    branch), and no M0 set for a copy may be followed by another such write before its copy."""
+    m0_write = re.compile(r"^(s_\w+)\s+m0\b")
+    kernel, in_asm, pending, bad, copies = None, False, None, [], 0
+    for i, line in enumerate(assembly):
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            kernel, pending = m.group(1), None
+        t = line.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if t.endswith(":") and not t.startswith(";"):
+            if pending is not None:
+                bad.append("%s: a label in line %d between the M0 of line %d and its copy" % (kernel, i + 1, pending))
+            pending = None
+            continue
+        if not _is_code(t):
+            continue
+        if m0_write.match(t):
+            if not in_asm:
+                bad.append("%s: line %d writes M0 outside an assembly statement (%s)" % (kernel, i + 1, t))
+            elif pending is not None:
+                bad.append("%s: M0 of line %d overwritten in line %d before its copy" % (kernel, pending, i + 1))
+            pending = i + 1
+            continue
+        if t.startswith("global_load_lds"):
+            copies += 1
+            if pending is None:
+                bad.append("%s: copy in line %d without an M0 set for it" % (kernel, i + 1))
+            pending = None
+            continue
+        if pending is not None and re.match(r"^(s_cbranch|s_branch|s_setpc|s_swappc|s_endpgm)", t):
+            bad.append("%s: line %d leaves the straight line between the M0 of line %d and its copy" % (kernel, i + 1, pending))
+            pending = None
+    assert copies > 100
+    assert not bad, "\n".join(bad[:20])
