@@ -15,7 +15,7 @@ FM_OK = 0
 FM_ERR_STRIDE = 3
 FM_ERR_ALIAS = 5
 # fm_knob values
-FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID, FM_KNOB_NO_SUB64, FM_KNOB_HALF, FM_KNOB_DIAG_LAST = 0, 1, 2, 3, 4, 5, 6
+FM_KNOB_GRID, FM_KNOB_KSPLIT, FM_KNOB_FAST_MIN_UNITS, FM_KNOB_NO_MID, FM_KNOB_NO_SUB64, FM_KNOB_HALF, FM_KNOB_DIAG_LAST, FM_KNOB_NO_TICKETS = 0, 1, 2, 3, 4, 5, 6, 7
 FM_BF16, FM_F16, FM_F32 = 0, 1, 2
 
 _DTYPE_CODE = {torch.bfloat16: FM_BF16, torch.float16: FM_F16, torch.float32: FM_F32}
@@ -143,7 +143,9 @@ def gemm_workspace(nbytes, device, stream=None):
     key = (torch.device(device).index, stream_ptr(device) if stream is None else stream)
     ws = _gemm_ws.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = _gemm_ws[key] = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        # zeroed once: its last 256 bytes hold the word the library counts sub-tile tickets in, which
+        # the library keeps in order from then on (garbage there costs speed, never correctness)
+        ws = _gemm_ws[key] = torch.zeros(nbytes, dtype=torch.uint8, device=device)
     return ws, ws.numel()
 
 

@@ -370,6 +370,10 @@ int fm_newtonschulz_batched_bf16(const void* const* G, int dtype, int batch, int
   void* gws = w + l.gemm;
   const size_t gws_bytes = l.total - l.gemm;
   hipStream_t hs = static_cast<hipStream_t>(stream);
+  // the last 256 bytes of the GEMM scratch hold the ticket word of the sub-tile rounds: whatever the
+  // caller's memory held there could pass for a launch number no launch ever reaches (the products
+  // would still be right, on the fixed assignment of sub-tiles), so it starts from zero
+  if (steps > 0 && gws_bytes >= 256 && launch_zero_words(w + l.total - 256, 32, hs)) return FM_ERR_LAUNCH;
   const bool tall = rows > cols;
   const bool padded = l.padded && steps > 0;
   const int M = padded ? l.M : (tall ? cols : rows), K = padded ? l.K : (tall ? rows : cols);

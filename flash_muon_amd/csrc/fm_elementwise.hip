@@ -252,6 +252,15 @@ int launch_scale_cast(const void* G, int dtype, int rows, int cols, int64_t ldg,
                                    T ? &T : nullptr, ldt, stream, rows, cols);
 }
 
+// ---- a few zero words (a fill launch rather than hipMemsetAsync, so that callers can be captured) ---
+__global__ void zero_words_kernel(unsigned long long* p, int n) {
+  if ((int)threadIdx.x < n) p[threadIdx.x] = 0ull;
+}
+int launch_zero_words(void* p, int n, hipStream_t stream) {
+  hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, stream, static_cast<unsigned long long*>(p), n < 64 ? n : 64);
+  return (int)hipGetLastError();
+}
+
 // ---- momentum + Nesterov ------------------------------------------------------------------------
 __device__ __forceinline__ float lerp_torch(float s, float e, float w) {
   // the two-branch form torch's lerp uses (weights below 0.5 interpolate from the start point)

@@ -273,7 +273,7 @@ struct KnobState {
   KnobState() {
     static const char* const names[kKnobCount] = {"FLASHMUON_GRID", "FLASHMUON_KSPLIT", "FLASHMUON_FAST_MIN_UNITS",
                                                   "FLASHMUON_NO_MID", "FLASHMUON_NO_SUB64", "FLASHMUON_HALF",
-                                                  "FLASHMUON_DIAG_LAST"};
+                                                  "FLASHMUON_DIAG_LAST", "FLASHMUON_NO_TICKETS"};
     for (int i = 0; i < kKnobCount; ++i) {
       const char* e = std::getenv(names[i]);
       v[i].store(e ? std::atoll(e) : -1, std::memory_order_relaxed);

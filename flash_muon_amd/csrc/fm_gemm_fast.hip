@@ -16,6 +16,8 @@
 
 #include <type_traits>
 #include <cstdlib>
+#include <atomic>
+#include <chrono>
 
 namespace fm {
 
@@ -1019,6 +1021,9 @@ struct FastArgs {
   int tail_slot0;       // first slot of the last round's sub-parts
   int reduce_tile0;     // first tile the second kernel has to finish
   int sub64;            // the left-over tiles are computed whole-k as 64x64 sub-tiles, 16 workgroups each
+  // Sub-tiles handed out in the order the workgroups arrive (below), or nullptr: sub-tile w to workgroup w.
+  unsigned long long* tickets;
+  unsigned long long epoch;   // this launch's number (48 bits, never 0)
   int half;             // the items are 128x256 half tiles, never cut (the NI == 2 kernels)
 };
 
@@ -1233,6 +1238,28 @@ __device__ __forceinline__ void diag_item(const GemmArgs& g, int m0, int n, unsi
 // flight.  The fragment reads of a stage are issued a stage ahead, behind the barrier that says it
 // has landed everywhere, and ride on the MFMAs of the stage before: wait, barrier, reads and MFMAs one
 // after the other cost 510 cycles a stage where the MFMAs take 128.
+// Tickets for the sub-tiles of one launch: a 64-bit word in the caller's workspace holds the launch's
+// number in its upper 48 bits and the count of tickets drawn in the lower 16.  Launch numbers grow, so
+// an atomic maximum with (number, 0), which every workgroup applies when it starts, turns whatever an
+// earlier launch left there into "none drawn" and leaves the word alone once this launch counts in it;
+// nothing has to be cleared beforehand.  A draw is one atomic add.  If it returns another launch's
+// number (the workspace held something larger than any launch number: never cleared, or written by
+// something else) there are no tickets, for anybody, and sub-tile w goes to workgroup w.  `total`
+// tickets are drawn in all (one per sub-tile, and one more per workgroup, that tells it to stop);
+// whoever draws the last one leaves the word at zero, so that a replay of the same launch from a HIP
+// graph finds it smaller than its number again.
+constexpr int kNoTickets = -1;
+__device__ __forceinline__ void open_tickets(unsigned long long* word, unsigned long long epoch) {
+  __hip_atomic_fetch_max(word, epoch << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int draw_ticket(unsigned long long* word, unsigned long long epoch, int total) {
+  const unsigned long long old = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if ((old >> 16) != epoch) return kNoTickets;
+  const int ticket = (int)(old & 0xffffull);
+  if (ticket == total - 1) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return ticket;
+}
+
 constexpr int SUB = 64;
 constexpr int SUB_OPER = SUB * ROWB;          // 64 rows of one operand stage: 8 KiB
 constexpr int SUB_STAGE = 2 * SUB_OPER;
@@ -1420,7 +1447,8 @@ template <bool F16, int MODE>
 __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n, float* slot, unsigned char* smem,
                                              const FragAddr16& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
                                              const bf16_t* gA, const bf16_t* gB, uint32_t ldsw, int row0, int col0,
-                                             int lane, int wave) {
+                                             int lane, int wave, unsigned long long* draw, unsigned long long epoch, int total,
+                                             int& ticket) {
   f32x4_t acc[8][8];   // started from zero by the first substep of the first stage
   {
     Frag16 f0, f1;
@@ -1477,6 +1505,9 @@ __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n
     wait_vmcnt<0>();
     __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
   }
+  // the last whole tile of a workgroup that goes on to sub-tiles: its first ticket is drawn here, so
+  // that the answer (a trip to memory and back, 3 us) arrives while the tile is written out
+  if (draw && threadIdx.x == 0) ticket = draw_ticket(draw, epoch, total);
   unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
   if (slot) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
     const EpiLds L = epi_lds(wave_lds);
@@ -1521,6 +1552,9 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   }
 
   const uint32_t ldsw = FM_LDS_ADDR(smem) + wave * 1024;   // where this wave's copies land inside a slot
+  if constexpr (NI == 4) {
+    if (p.tickets != nullptr && tid == 0) open_tickets(p.tickets, p.epoch);
+  }
 
   // whole tiles (NI == 4) run on 16x16x32 MFMAs: row = lane % 16 of a fragment's 16 LDS rows, k quarter = lane / 16
   FragAddr16 fa16;
@@ -1553,6 +1587,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     for (int ks = 0; ks < 4; ++ks) fa.b[i][ks] = (bo ^ (ks << 5)) + b_slot_off(0);
   }
 
+  int first_ticket = kNoTickets;   // thread 0: the ticket drawn ahead of the sub-tile round
   for (int round = 0; round <= p.rounds; ++round) {
     int item, slot_id, kb, ke;
     if (round < p.rounds) {
@@ -1566,11 +1601,44 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
       kb = 0;
       ke = p.nk;
     } else if (NI == 4 && p.sub64) {
-      if (w >= p.rem * 16) break;
-      int sbi, sti, stj;
-      tile_at(p.g, p.rounds * p.grid + (w >> 4), sbi, sti, stj);
-      const GemmArgs sg = batch_view(p.g, sbi);
-      sub64_tile<F16>(sg, sti, stj, (w >> 2) & 3, w & 3, p.nk, smem, lane, wave);
+      if (p.tickets == nullptr) {   // sub-tile w to workgroup w
+        if (w >= p.rem * 16) break;
+        int sbi, sti, stj;
+        tile_at(p.g, p.rounds * p.grid + (w >> 4), sbi, sti, stj);
+        const GemmArgs sg = batch_view(p.g, sbi);
+        sub64_tile<F16>(sg, sti, stj, (w >> 2) & 3, w & 3, p.nk, smem, lane, wave);
+        break;
+      }
+      // The workgroups do not leave the last full round together: the XCDs of one chip differ by
+      // several per cent over two rounds.  So the sub-tiles are taken by ticket, in the order the
+      // workgroups get here, and a workgroup that is done early takes another.
+      // (when the tiles left over are all diagonal ones, only the 10 sub-tiles on or above the
+      // diagonal of each have a ticket: the other 6 are their mirror images)
+      const int per_tile = p.g.diag_last > 0 ? 10 : 16;
+      for (bool first = true;; first = false) {
+        __syncthreads();   // nobody still uses the first word of LDS, or the ring, for the sub-tile before
+        if (tid == 0)   // (the first ticket was drawn behind the main loop of the last whole tile)
+          *reinterpret_cast<volatile int*>(smem) = first ? first_ticket : draw_ticket(p.tickets, p.epoch, p.rem * per_tile + p.grid);
+        __syncthreads();
+        int t = __builtin_amdgcn_readfirstlane(*reinterpret_cast<volatile int*>(smem));
+        int tile, si, sj;
+        if (t == kNoTickets) {
+          if (w >= p.rem * 16) break;
+          tile = w >> 4; si = (w >> 2) & 3; sj = w & 3;
+        } else {
+          if (t >= p.rem * per_tile) break;
+          tile = t / per_tile;
+          const int idx = t - tile * per_tile;
+          if (per_tile == 10) tri_decode(idx, 4, si, sj);
+          else { si = idx >> 2; sj = idx & 3; }
+        }
+        __syncthreads();   // everybody has read the ticket before the copies overwrite it
+        int sbi, sti, stj;
+        tile_at(p.g, p.rounds * p.grid + tile, sbi, sti, stj);
+        const GemmArgs sg = batch_view(p.g, sbi);
+        sub64_tile<F16>(sg, sti, stj, si, sj, p.nk, smem, lane, wave);
+        if (t == kNoTickets) break;
+      }
       break;
     } else {
       if (w >= p.rem * p.split) break;
@@ -1617,7 +1685,9 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     if constexpr (NI == 4) {   // whole tiles, or parts of them along k
       const bool diag = g.symmetric && ti == tj;
       float* const slot = n != p.nk ? p.partials + (size_t)slot_id * PART_FLOATS : nullptr;
-      whole_tile16<F16, MODE>(g, diag, n, slot, smem, fa16, voA, voB, gA, gB, ldsw, m0 + wm * 128, n0 + wn * 128, lane, wave);
+      const bool draws = p.sub64 && p.tickets != nullptr && round == p.rounds - 1;
+      whole_tile16<F16, MODE>(g, diag, n, slot, smem, fa16, voA, voB, gA, gB, ldsw, m0 + wm * 128, n0 + wn * 128, lane, wave,
+                              draws ? p.tickets : nullptr, p.epoch, p.rem * (p.g.diag_last > 0 ? 10 : 16) + p.grid, first_ticket);
       __syncthreads();   // the next tile's copies land in the memory the staging just used
     } else {   // 128x256 half tiles: 32x32x16 MFMAs
 
@@ -1957,6 +2027,16 @@ __global__ __launch_bounds__(256) void gemm_nt_mid_reduce_kernel(GemmArgs gb, Mi
 
 }  // namespace
 
+constexpr size_t kTicketBytes = 256;   // what a workspace holds behind its partial-tile slots
+// where this process starts numbering its launches: 2^30 .. 2^46, from the clock and the address space
+static unsigned long long first_launch_number() {
+  const unsigned long long t = (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count();
+  const unsigned long long a = (unsigned long long)reinterpret_cast<uintptr_t>(&kTicketBytes);
+  unsigned long long x = t ^ (a * 0x9E3779B97F4A7C15ull);
+  x ^= x >> 29; x *= 0xBF58476D1CE4E5B9ull; x ^= x >> 32;
+  return (1ull << 30) + (x & ((1ull << 46) - 1));
+}
+
 // Too few tiles for one round (M = 4096 gives 136 symmetric tiles) and a long k: every tile is cut
 // along k into as many base parts as fill the chip, each at least 64 stages long so that the fp32
 // round trip of its partial tile stays a small part of its time.
@@ -2200,7 +2280,9 @@ size_t gemm_fast_workspace_bytes(int Ma, int Nb, int batch) {
     if (slots > need) need = slots;
   }
   const size_t fast_need = (size_t)need * PART_FLOATS * sizeof(float);
-  return fast_need > mid_need ? fast_need : mid_need;
+  // (the ticket word of the sub-tile rounds lies behind the slots; a product of more tiles than CUs
+  // that cuts nothing still has it)
+  return (fast_need > mid_need ? fast_need : mid_need) + kTicketBytes;
 }
 
 int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) {
@@ -2211,7 +2293,9 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   FastArgs f;
   f.g = a;
   f.nk = a.Kc / BKF;
-  const long long have = ws ? (long long)(ws_bytes / (PART_FLOATS * sizeof(float))) : 0;
+  // the last 256 bytes of a workspace are the ticket word's (below), the partial-tile slots lie in front of them
+  const size_t slot_bytes = ws && ws_bytes >= kTicketBytes ? ws_bytes - kTicketBytes : 0;
+  const long long have = (long long)(slot_bytes / (PART_FLOATS * sizeof(float)));
   fast_schedule(a.num_tiles, f.nk, have < kMaxSlots ? have : kMaxSlots, f);
   f.half = 0;
   int grid = cu_count() < kMaxGrid ? cu_count() : kMaxGrid;
@@ -2246,6 +2330,19 @@ int launch_gemm_fast(GemmArgs a, void* ws, size_t ws_bytes, hipStream_t stream) 
   if (f.sub64 && f.rounds > 0 && a.symmetric && a.batch == 1 && f.rem <= a.tiles_m && knob(kKnobDiagLast) != 0)
     f.g.diag_last = f.rem;
   f.partials = static_cast<float*>(ws);
+  // The sub-tiles behind full rounds go out by ticket when there is a workspace to count in: the
+  // word is the first of its last 256-byte block.  65535 tickets at most.  Launch numbers start at a
+  // value of this process's own (so that a word another process left in the same memory does not
+  // carry a number this one will reach) and stay below 2^47.
+  f.tickets = nullptr;
+  f.epoch = 0;
+  if (f.sub64 && f.rounds > 0 && ws && ws_bytes >= 2 * kTicketBytes && f.rem * 16 + f.grid < 65536 && knob(kKnobNoTickets) <= 0) {
+    // (fewer than 65536 tickets; whether a tile has 10 or 16 is the kernel's business)
+    static std::atomic<unsigned long long> launches{first_launch_number()};
+    f.epoch = launches.fetch_add(1, std::memory_order_relaxed) & 0x7fffffffffffull;
+    if (f.epoch != 0)
+      f.tickets = reinterpret_cast<unsigned long long*>(static_cast<unsigned char*>(ws) + (ws_bytes / kTicketBytes - 1) * kTicketBytes);
+  }
   if (f.half) {
     if (a.elem == kElemF16) hipLaunchKernelGGL((gemm_nt_rounds_kernel<true, 0, 2>), dim3(f.grid), dim3(256), 0, stream, f);
     else if (!a.E) hipLaunchKernelGGL((gemm_nt_rounds_kernel<false, 0, 2>), dim3(f.grid), dim3(256), 0, stream, f);

@@ -21,7 +21,7 @@ constexpr int kErrWorkspace = -2;     // the schedule needs more partial-tile sl
 // Tuning knobs (fm_set_knob, include/flashmuon.h); the FLASHMUON_* environment variables of the same
 // names give their initial values, read once when the library is first used.  A negative value
 // means "decide automatically".
-constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobNoSub64 = 4, kKnobHalf = 5, kKnobDiagLast = 6, kKnobCount = 7;
+constexpr int kKnobGrid = 0, kKnobKsplit = 1, kKnobFastMinUnits = 2, kKnobNoMid = 3, kKnobNoSub64 = 4, kKnobHalf = 5, kKnobDiagLast = 6, kKnobNoTickets = 7, kKnobCount = 8;
 long long knob(int which);
 int set_knob(int which, long long value);
 // compute units of the current device (queried once per device)
@@ -154,6 +154,9 @@ int launch_momentum_nesterov(void* g, void* buf, int dtype, int64_t n, float w_b
                              int nesterov, hipStream_t stream);
 int launch_weight_update(void* p, int p_dtype, const bf16_t* u, int64_t n, float decay_mul,
                          float alpha, hipStream_t stream);
+
+// n (at most 64) 64-bit words at p set to zero by a one-block launch
+int launch_zero_words(void* p, int n, hipStream_t stream);
 
 constexpr int kSumsqBlocks = 1024;   // partial sums written by the first reduction stage
 

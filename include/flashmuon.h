@@ -58,8 +58,8 @@ FM_API const char* fm_version(void);
 
 /* Tuning knobs, for experiments and for tests that have to reach a particular schedule.  A
  * negative value gives the decision back to the library.  The environment variables
- * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS, FLASHMUON_NO_MID, FLASHMUON_NO_SUB64, FLASHMUON_HALF
- * and FLASHMUON_DIAG_LAST set the initial
+ * FLASHMUON_GRID, FLASHMUON_KSPLIT, FLASHMUON_FAST_MIN_UNITS, FLASHMUON_NO_MID, FLASHMUON_NO_SUB64, FLASHMUON_HALF,
+ * FLASHMUON_DIAG_LAST and FLASHMUON_NO_TICKETS set the initial
  * values; they are read once, when the library is first used, never per call.  No counterpart in
  * the reference (its tuning is Triton's autotune table, flash_muon/matmul_transpose_triton.py:6-18).
  */
@@ -74,9 +74,11 @@ enum fm_knob {
                                   sixteenth as many 256x256 tiles as workgroups on them (by estimate otherwise) */
   FM_KNOB_HALF = 5,            /* 1: always, 0: never run the 256x256 schedule on 128x256 half tiles (taken by
                                   itself when all of them fit into one round of workgroups) */
-  FM_KNOB_DIAG_LAST = 6        /* 0: the tiles left after the last full round of a symmetric product are the
+  FM_KNOB_DIAG_LAST = 6,       /* 0: the tiles left after the last full round of a symmetric product are the
                                   last of the blocked tile order, whatever they are (otherwise: diagonal tiles,
                                   which need one operand panel each and 10 of their 16 sub-tiles) */
+  FM_KNOB_NO_TICKETS = 7       /* 1: sub-tile w of the last round goes to workgroup w even where a workspace is
+                                  there to hand them out in (otherwise: in the order the workgroups arrive) */
 };
 FM_API int fm_set_knob(int knob, long long value);
 

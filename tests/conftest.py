@@ -23,7 +23,7 @@ def lib():
 
 
 KNOBS = {"FLASHMUON_GRID": 0, "FLASHMUON_KSPLIT": 1, "FLASHMUON_FAST_MIN_UNITS": 2, "FLASHMUON_NO_MID": 3,
-         "FLASHMUON_NO_SUB64": 4, "FLASHMUON_HALF": 5, "FLASHMUON_DIAG_LAST": 6}
+         "FLASHMUON_NO_SUB64": 4, "FLASHMUON_HALF": 5, "FLASHMUON_DIAG_LAST": 6, "FLASHMUON_NO_TICKETS": 7}
 
 
 @pytest.fixture
