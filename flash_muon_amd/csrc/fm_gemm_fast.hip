@@ -1242,19 +1242,20 @@ __device__ __forceinline__ void diag_item(const GemmArgs& g, int m0, int n, unsi
 // number in its upper 48 bits and the count of tickets drawn in the lower 16.  Launch numbers grow, so
 // an atomic maximum with (number, 0), which every workgroup applies when it starts, turns whatever an
 // earlier launch left there into "none drawn" and leaves the word alone once this launch counts in it;
-// nothing has to be cleared beforehand.  A draw is one atomic add.  If it returns another launch's
-// number (the workspace held something larger than any launch number: never cleared, or written by
-// something else) there are no tickets, for anybody, and sub-tile w goes to workgroup w.  `total`
-// tickets are drawn in all (one per sub-tile, and one more per workgroup, that tells it to stop);
-// whoever draws the last one leaves the word at zero, so that a replay of the same launch from a HIP
-// graph finds it smaller than its number again.
+// nothing has to be cleared beforehand.  What the maximum returns tells the workgroup whether there
+// are tickets: if the word held something beyond this launch's numbers (never cleared, or written by
+// something else) it stays as it is, nobody ever draws, and sub-tile w goes to workgroup w; every
+// workgroup sees the same.  A draw is one atomic add.  `total` tickets are drawn in all (one per
+// sub-tile, and one more per workgroup, that tells it to stop); whoever draws the last one leaves the
+// word at zero, so that a replay of the same launch from a HIP graph finds it below its number again.
 constexpr int kNoTickets = -1;
-__device__ __forceinline__ void open_tickets(unsigned long long* word, unsigned long long epoch) {
-  __hip_atomic_fetch_max(word, epoch << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ bool open_tickets(unsigned long long* word, unsigned long long epoch) {
+  const unsigned long long old = __hip_atomic_fetch_max(word, epoch << 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return old < ((epoch + 1) << 16);
 }
 __device__ __forceinline__ int draw_ticket(unsigned long long* word, unsigned long long epoch, int total) {
   const unsigned long long old = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  if ((old >> 16) != epoch) return kNoTickets;
+  if ((old >> 16) != epoch) return kNoTickets;   // (not reached: the word was opened for this launch)
   const int ticket = (int)(old & 0xffffull);
   if (ticket == total - 1) __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return ticket;
@@ -1552,8 +1553,9 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
   }
 
   const uint32_t ldsw = FM_LDS_ADDR(smem) + wave * 1024;   // where this wave's copies land inside a slot
+  bool tickets_live = false;   // thread 0: the sub-tile round of this launch hands out tickets
   if constexpr (NI == 4) {
-    if (p.tickets != nullptr && tid == 0) open_tickets(p.tickets, p.epoch);
+    if (p.tickets != nullptr && tid == 0) tickets_live = open_tickets(p.tickets, p.epoch);
   }
 
   // whole tiles (NI == 4) run on 16x16x32 MFMAs: row = lane % 16 of a fragment's 16 LDS rows, k quarter = lane / 16
@@ -1685,7 +1687,7 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     if constexpr (NI == 4) {   // whole tiles, or parts of them along k
       const bool diag = g.symmetric && ti == tj;
       float* const slot = n != p.nk ? p.partials + (size_t)slot_id * PART_FLOATS : nullptr;
-      const bool draws = p.sub64 && p.tickets != nullptr && round == p.rounds - 1;
+      const bool draws = p.sub64 && p.tickets != nullptr && round == p.rounds - 1 && tickets_live;
       whole_tile16<F16, MODE>(g, diag, n, slot, smem, fa16, voA, voB, gA, gB, ldsw, m0 + wm * 128, n0 + wn * 128, lane, wave,
                               draws ? p.tickets : nullptr, p.epoch, p.rem * (p.g.diag_last > 0 ? 10 : 16) + p.grid, first_ticket);
       __syncthreads();   // the next tile's copies land in the memory the staging just used

@@ -302,3 +302,78 @@ def test_operands_and_outputs_across_a_4gib_boundary(lib, knobs):
     Pb.copy_(Pm)
     got = gpu_util.gemm_axpby(lib, Pb, Xs, 2.0)
     assert torch.equal(got[0], Xo) and torch.equal(got[1], XoT)
+
+
+def _ticket_word(ws):
+    """The 64-bit word the sub-tile tickets are counted in: the first of the workspace's last 256 bytes."""
+    nb = ws.numel() // 256 * 256
+    return ws[nb - 256: nb - 248].view(torch.int64)
+
+
+@pytest.mark.parametrize("M,K,grid", [(2048, 1024, 34), (2304, 512, 43), (4352, 128, 144)])
+def test_sub_tiles_by_ticket_whatever_the_workspace_holds(lib, knobs, M, K, grid):
+    """With a workspace the sub-tiles of the last round are handed out by ticket (fewer workgroups than
+    sub-tiles here, so workgroups come back for more).  The ticket word may hold anything when the call
+    starts: zero, an earlier launch's count, a value smaller or larger than any launch number (the last
+    means no tickets: sub-tile w to workgroup w), or what a call that cut its tiles along k wrote there.
+    Every sub-tile is computed exactly once each time, and the word is left at zero, or alone."""
+    knobs("FLASHMUON_GRID", grid)
+    X = _ints((M, K), M + K + grid)
+    want = _exact(X.double() @ X.double().T)
+    Xd = X.to(DEV)
+    ws = torch.zeros(lib.fm_gemm_workspace_bytes(M, M), dtype=torch.uint8, device=DEV)
+    word = _ticket_word(ws)
+
+    def run():
+        Y = torch.full((M, M), float("nan"), dtype=torch.bfloat16, device=DEV)
+        st = lib.fm_syrk_bf16(Xd.data_ptr(), K, Y.data_ptr(), M, 1, M, K, ws.data_ptr(), ws.numel(), gpu_util._stream(Xd))
+        assert st == 0
+        torch.cuda.synchronize()
+        assert torch.equal(Y.cpu(), want)
+
+    for start in (0, 5, 1 << 20, (1 << 62) + 12345, -1, -(1 << 40)):
+        word.fill_(start)
+        run()
+        left = int(word.item())
+        if 0 <= start < (1 << 46):
+            assert left == 0, (start, left)          # below every launch number: tickets, and the last one clears the word
+        else:
+            assert left == (start if start >= 0 else start), (start, left)   # beyond them: no tickets, the word is left alone
+        run()                                        # and again over what that call left
+    # a call of the same shape that cuts its left-over tiles along k fills the slots in front of the word
+    word.fill_(0)
+    knobs("FLASHMUON_NO_SUB64", 1)
+    run()
+    knobs("FLASHMUON_NO_SUB64", -1)
+    run()
+    assert int(word.item()) == 0
+    # no tickets at all by knob: same result
+    knobs("FLASHMUON_NO_TICKETS", 1)
+    word.fill_(77)
+    run()
+    assert int(word.item()) == 77
+
+
+def test_sub_tiles_by_ticket_in_a_graph(lib, knobs):
+    """A captured call carries its launch number with it: every replay finds the word at zero (the last
+    ticket of the replay before cleared it) and counts from there."""
+    knobs("FLASHMUON_GRID", 34)
+    M, K = 2048, 512
+    X = torch.randn(M, K, generator=torch.Generator().manual_seed(3)).bfloat16().to(DEV)
+    ws = torch.zeros(lib.fm_gemm_workspace_bytes(M, M), dtype=torch.uint8, device=DEV)
+    Y = torch.empty(M, M, dtype=torch.bfloat16, device=DEV)
+    want = gpu_util.syrk(lib, X)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        st = lib.fm_syrk_bf16(X.data_ptr(), K, Y.data_ptr(), M, 1, M, K, ws.data_ptr(), ws.numel(),
+                              torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+    for i in range(4):
+        Y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(Y, want), "replay %d" % i
+        assert int(_ticket_word(ws).item()) == 0
+        assert torch.equal(gpu_util.syrk(lib, X), want)   # eager calls in between, with a workspace of their own
