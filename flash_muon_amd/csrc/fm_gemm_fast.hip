@@ -45,12 +45,6 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
 
-#define FM_MFMA(i, j, FA, FB) acc[i][j] = mfma_32x32x16<F16>(FA[i], FB[j], acc[i][j])
-
-// NI: rows of 32x32 MFMA tiles per wave.  4: a wave computes 128x128 of a 256x256 tile; 2: 64x128
-// of a 128x256 half tile (operand A is then half as tall and uses half of each of its slots).
-template <int NI> struct Frag { bf16x8_t a[NI], b[4]; };
-
 // LDS during the main loop: three stages of operand A and two of operand B, 32 KiB each, in the
 // order A0 A1 B0 B1 A2.  Stage s of A sits in A slot s % 3, stage s of B in B slot s % 2.  A
 // ds_read takes a 16-bit immediate offset, so one address register reaches two neighbouring slots:
@@ -59,23 +53,6 @@ template <int NI> struct Frag { bf16x8_t a[NI], b[4]; };
 // the second one by its own issue time).
 __host__ __device__ constexpr int a_slot_off(int slot) { return slot == 2 ? 4 * OPER_BYTES : slot * OPER_BYTES; }
 __host__ __device__ constexpr int b_slot_off(int slot) { return (2 + slot) * OPER_BYTES; }
-
-// per-lane LDS byte addresses of the fragments: [window][fragment][k16 substep]
-template <int NI> struct FragAddr {
-  uint32_t a_lo[NI][4];  // A rows, slots 0 and 1 (offset 0 / OPER_BYTES)
-  uint32_t a_hi[NI][4];  // A rows, slot 2
-  uint32_t b[4][4];      // B rows, B slots 0 and 1 (offset 0 / OPER_BYTES from the window at 64 KiB)
-};
-
-template <int ASLOT, int NI>
-__device__ __forceinline__ bf16x8_t read_a(const unsigned char* smem, const FragAddr<NI>& fa, int i, int ks) {
-  if constexpr (ASLOT == 2) return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_hi[i][ks]);
-  else return *reinterpret_cast<const bf16x8_t*>(smem + fa.a_lo[i][ks] + ASLOT * OPER_BYTES);
-}
-template <int BSLOT, int NI>
-__device__ __forceinline__ bf16x8_t read_b(const unsigned char* smem, const FragAddr<NI>& fa, int j, int ks) {
-  return *reinterpret_cast<const bf16x8_t*>(smem + fa.b[j][ks] + BSLOT * OPER_BYTES);
-}
 
 // one global -> LDS copy with the destination given as an offset from the wave's copy base.
 // (s_add_i32 writes SCC: without the clobber the compiler keeps the carry of a 64-bit pointer
@@ -95,71 +72,6 @@ __device__ __forceinline__ void dma16_m0(uint32_t lds_base, int off) {
 }
 __device__ __forceinline__ void dma16_go(uint32_t voff, const void* sbase) {
   asm volatile("global_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase) : "memory");
-}
-
-// The 4 NI MFMAs of k16 substep KS of the stage in (ASLOT, BSLOT).  The NI + 4 fragment reads of
-// the next substep ride on the first ones, and copies Q0 .. Q1-1 of operand A of the stage two
-// ahead (into the A slot that the previous stage has left) go out between the others, so that the
-// memory pipeline sees an even stream of requests and each of these copies has almost two stages
-// to land.
-// FIRST: the first substep of a tile, which starts its accumulators from zero instead of having
-// the registers cleared beforehand.
-template <bool F16, int NI, int ASLOT, int BSLOT, int KS, int Q0, int Q1, bool FIRST = false, int NR>
-__device__ __forceinline__ void phase(f32x16_t (&acc)[NR][4], const Frag<NI>& cur, Frag<NI>& nxt,
-                                      const unsigned char* smem, const FragAddr<NI>& fa,
-                                      const uint32_t (&voA)[2 * NI], const bf16_t* gA, uint32_t ldsw) {
-  constexpr int AFREE = (ASLOT + 2) % 3;
-  constexpr int DQ0 = NI == 4 ? 9 : 6, DSTEP = NI == 4 ? 2 : 1;   // where the copies go: after the reads
-#pragma unroll
-  for (int q = 0; q < 4 * NI; ++q) {
-    if (q < NI) nxt.a[q] = read_a<ASLOT>(smem, fa, q, KS + 1);
-    else if (q < NI + 4) nxt.b[q - NI] = read_b<BSLOT>(smem, fa, q - NI, KS + 1);
-    if (q >= DQ0 && (q - DQ0) % DSTEP == 0 && Q0 + (q - DQ0) / DSTEP < Q1)
-      dma16o(voA[Q0 + (q - DQ0) / DSTEP], gA, ldsw, a_slot_off(AFREE) + (Q0 + (q - DQ0) / DSTEP) * 4096);
-    if constexpr (FIRST) {
-      const f32x16_t zero = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-      acc[q >> 2][q & 3] = mfma_32x32x16<F16>(cur.a[q >> 2], cur.b[q & 3], zero);
-    } else {
-      FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-}
-
-// Last substep of a stage.  Before it every wave waits for its copies of the next stage (all but
-// the 2 NI newest, which belong to the stage after) and, at the barrier, for everybody else's; then
-// the MFMAs run interleaved with the 8 copies of operand B two stages ahead, into the B slot
-// this stage has just left, and with the first fragment reads of the next stage.
-template <bool F16, int NI, int ASLOT, int BSLOT, int NR>
-__device__ __forceinline__ void tail_phase(f32x16_t (&acc)[NR][4], const Frag<NI>& cur, Frag<NI>& nxt,
-                                           const unsigned char* smem, const FragAddr<NI>& fa,
-                                           const uint32_t (&voB)[8], const bf16_t* gB, uint32_t ldsw) {
-  constexpr int ANEXT = (ASLOT + 1) % 3, BNEXT = BSLOT ^ 1;
-  constexpr int BSTEP = NI / 2;   // MFMAs per copy of operand B
-  // (the fragment reads of this stage were issued a substep ago; lgkmcnt(0) makes it formal that
-  // nobody still reads the slots that are about to be refilled)
-  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" :: "n"(2 * NI) : "memory");
-#pragma unroll
-  for (int q = 0; q < 4 * NI; ++q) {
-    if (q % BSTEP == 0) dma16o(voB[q / BSTEP], gB, ldsw, b_slot_off(BSLOT) + (q / BSTEP) * 4096);
-    if (q < NI) nxt.a[q] = read_a<ANEXT>(smem, fa, q, 0);
-    else if (q < NI + 4) nxt.b[q - NI] = read_b<BNEXT>(smem, fa, q - NI, 0);
-    FM_MFMA(q >> 2, q & 3, cur.a, cur.b);
-    __builtin_amdgcn_sched_barrier(0);
-  }
-}
-
-// one k stage: the stage in (ASLOT, BSLOT) is multiplied, operand A of the stage two ahead is
-// copied during the first three substeps and operand B of it during the last
-template <bool F16, int NI, int ASLOT, int BSLOT, bool FIRST = false, int NR>
-__device__ __forceinline__ void stage(f32x16_t (&acc)[NR][4], Frag<NI>& f0, Frag<NI>& f1, const unsigned char* smem,
-                                      const FragAddr<NI>& fa, const uint32_t (&voA)[2 * NI], const uint32_t (&voB)[8],
-                                      const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
-  constexpr int Q1 = NI == 4 ? 3 : 2, Q2 = NI == 4 ? 6 : 3;   // the 2 NI copies of operand A over three substeps
-  phase<F16, NI, ASLOT, BSLOT, 0, 0, Q1, FIRST>(acc, f0, f1, smem, fa, voA, nA, ldsw);
-  phase<F16, NI, ASLOT, BSLOT, 1, Q1, Q2>(acc, f1, f0, smem, fa, voA, nA, ldsw);
-  phase<F16, NI, ASLOT, BSLOT, 2, Q2, 2 * NI>(acc, f0, f1, smem, fa, voA, nA, ldsw);
-  tail_phase<F16, NI, ASLOT, BSLOT>(acc, f1, f0, smem, fa, voB, nB, ldsw);
 }
 
 // ---- whole tiles on 16x16x32 MFMAs --------------------------------------------------------------
@@ -193,7 +105,8 @@ __device__ __forceinline__ f32x4_t mfma_16x16x32(bf16x8_t a, bf16x8_t b, f32x4_t
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-struct Frag16 { bf16x8_t a[8], b[8]; };
+// NA: 16-row fragments of operand A per wave: 8 for a whole tile (128 rows), 4 for a 128x256 half tile (64 rows)
+template <int NA> struct Frag16 { bf16x8_t a[NA], b[8]; };
 // per-lane LDS byte addresses of fragment 0 for k32 substep kk: operand A in A slots 0 and 1
 // (a_lo, + OPER_BYTES) and in A slot 2 (a_hi), operand B in B slots 0 and 1
 struct FragAddr16 { uint32_t a_lo[2], a_hi[2], b[2]; };
@@ -208,16 +121,16 @@ __device__ __forceinline__ bf16x8_t read_b16(const unsigned char* smem, const Fr
   return *reinterpret_cast<const bf16x8_t*>(smem + fa.b[kk] + BSLOT * OPER_BYTES + j * 2048);
 }
 
-// The 64 MFMAs of k32 substep KK of the stage in (ASLOT, BSLOT).  The 16 fragment reads of the
-// next substep (the second half of this stage, or the first half of the next one) ride on the first 32
-// of them, in the order the next substep needs them.  During substep 0 the 8 copies of operand A of
-// the stage two ahead go out, into the A slot the previous stage has left; during the first half of
-// substep 1, behind the barrier of the stage, the 8 copies of operand B of that stage, into the B
-// slot this stage has just read for the last time.
-template <bool F16, int ASLOT, int BSLOT, int KK, bool FIRST>
-__device__ __forceinline__ void substep16(f32x4_t (&acc)[8][8], const Frag16& cur, Frag16& nxt,
+// The 8 NA MFMAs of k32 substep KK of the stage in (ASLOT, BSLOT).  The NA + 8 fragment reads of the
+// next substep (the second half of this stage, or the first half of the next one) ride on the first
+// 2 (NA + 8) of them, in the order the next substep needs them.  During substep 0 the NA copies of
+// operand A of the stage two ahead go out, into the A slot the previous stage has left; during the
+// first 32 MFMAs of substep 1, behind the barrier of the stage, the 8 copies of operand B of that
+// stage, into the B slot this stage has just read for the last time.
+template <bool F16, int NA, int ASLOT, int BSLOT, int KK, bool FIRST>
+__device__ __forceinline__ void substep16(f32x4_t (&acc)[NA][8], const Frag16<NA>& cur, Frag16<NA>& nxt,
                                           const unsigned char* smem, const FragAddr16& fa,
-                                          const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                          const uint32_t (&voA)[NA], const uint32_t (&voB)[8],
                                           const bf16_t* gA, const bf16_t* gB, uint32_t ldsw) {
   constexpr int AFREE = (ASLOT + 2) % 3, ANEXT = (ASLOT + 1) % 3, BNEXT = BSLOT ^ 1;
   // every fragment of this substep was asked for half a substep ago: one wait for all of them, said
@@ -225,9 +138,9 @@ __device__ __forceinline__ void substep16(f32x4_t (&acc)[8][8], const Frag16& cu
   // of the first use of each
   if constexpr (KK == 0) __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0)
 #pragma unroll
-  for (int q = 0; q < 64; ++q) {
-    if ((q & 1) == 0 && q < 32) {
-      const int t = q >> 1;   // read t of the next substep: a0, b0 .. b7, a1 .. a7
+  for (int q = 0; q < 8 * NA; ++q) {
+    if ((q & 1) == 0 && q < 2 * (NA + 8)) {
+      const int t = q >> 1;   // read t of the next substep: a0, b0 .. b7, a1 .. a(NA - 1)
       if constexpr (KK == 0) {
         if (t == 0) nxt.a[0] = read_a16<ASLOT>(smem, fa, 0, 1);
         else if (t <= 8) nxt.b[t - 1] = read_b16<BSLOT>(smem, fa, t - 1, 1);
@@ -257,16 +170,16 @@ __device__ __forceinline__ void substep16(f32x4_t (&acc)[8][8], const Frag16& cu
 }
 
 // One k stage.  At the barrier between its substeps every wave has waited for its copies of the
-// next stage (all but the 8 newest, operand A of the stage after), and every fragment read of this
+// next stage (all but the NA newest, operand A of the stage after), and every fragment read of this
 // stage has returned, so that its B slot may be refilled.
-template <bool F16, int ASLOT, int BSLOT, bool FIRST = false>
-__device__ __forceinline__ void stage16(f32x4_t (&acc)[8][8], Frag16& f0, Frag16& f1, const unsigned char* smem,
-                                        const FragAddr16& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+template <bool F16, int NA, int ASLOT, int BSLOT, bool FIRST = false>
+__device__ __forceinline__ void stage16(f32x4_t (&acc)[NA][8], Frag16<NA>& f0, Frag16<NA>& f1, const unsigned char* smem,
+                                        const FragAddr16& fa, const uint32_t (&voA)[NA], const uint32_t (&voB)[8],
                                         const bf16_t* nA, const bf16_t* nB, uint32_t ldsw) {
-  substep16<F16, ASLOT, BSLOT, 0, FIRST>(acc, f0, f1, smem, fa, voA, voB, nA, nB, ldsw);
-  __builtin_amdgcn_s_waitcnt(0x0078);   // vmcnt(8) lgkmcnt(0)
+  substep16<F16, NA, ASLOT, BSLOT, 0, FIRST>(acc, f0, f1, smem, fa, voA, voB, nA, nB, ldsw);
+  __builtin_amdgcn_s_waitcnt(0x0070 | NA);   // vmcnt(NA) lgkmcnt(0)
   asm volatile("s_barrier" ::: "memory");
-  substep16<F16, ASLOT, BSLOT, 1, false>(acc, f1, f0, smem, fa, voA, voB, nA, nB, ldsw);
+  substep16<F16, NA, ASLOT, BSLOT, 1, false>(acc, f1, f0, smem, fa, voA, voB, nA, nB, ldsw);
 }
 
 // ---- a diagonal tile of a symmetric product as one item of the half-tile schedule ---------------
@@ -374,25 +287,8 @@ __device__ __forceinline__ EpiLds epi_lds(unsigned char* wave_base) {
 // float index of row r (0..31) of column c (0..127) in F
 __device__ __forceinline__ int qf_idx(int c, int r) { return c * QF_PITCH + (r ^ (((c >> 3) & 7) << 2)); }
 
-// accumulators of MFMA tile row i -> F.  Register 4q+e of lane l in MFMA tile (i, j) is row
-// 8q + 4(l/32) + e, column 32j + l%32 of the quarter: four consecutive rows of one column.
-template <int I, int NI>
-__device__ __forceinline__ void stage_store(const f32x16_t (&acc)[NI][4], float* F, int lane) {
-  const int c = lane & 31, rg = 4 * (lane >> 5);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    // (sub-vectors, not element reads: see the note on identical element reads at epilogue_regs)
-    const f32x16_t a = acc[I][j];
-    float* const dst = F + (32 * j + c) * QF_PITCH;
-    const int x = ((32 * j + c) >> 3 & 7) << 2;
-    *reinterpret_cast<f32x4_t*>(dst + ((0 + rg) ^ x)) = __builtin_shufflevector(a, a, 0, 1, 2, 3);
-    *reinterpret_cast<f32x4_t*>(dst + ((8 + rg) ^ x)) = __builtin_shufflevector(a, a, 4, 5, 6, 7);
-    *reinterpret_cast<f32x4_t*>(dst + ((16 + rg) ^ x)) = __builtin_shufflevector(a, a, 8, 9, 10, 11);
-    *reinterpret_cast<f32x4_t*>(dst + ((24 + rg) ^ x)) = __builtin_shufflevector(a, a, 12, 13, 14, 15);
-  }
-}
-
-// one MFMA tile of the accumulators -> columns 32 ct .. +31 of a staged quarter (as stage_store)
+// One 32x32 MFMA tile of the accumulators -> columns 32 ct .. +31 of a staged quarter: register 4q+e of
+// lane l is row 8q + 4(l/32) + e, column l%32 of the tile, four consecutive rows of one column.
 __device__ __forceinline__ void stage_tile(const f32x16_t& a, float* F, int ct, int lane) {
   const int col = 32 * ct + (lane & 31), rg = 4 * (lane >> 5);
   float* const dst = F + col * QF_PITCH;
@@ -834,7 +730,7 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
 }
 
 // ---- write-out of a whole tile from the 16x16 accumulator tiles ---------------------------------
-// The wave's block is 128 rows x 128 columns at (row0, col0); per 32x32 sub-block (I, J) a lane (n =
+// The wave's block is 16 NA rows x 128 columns at (row0, col0); per 32x32 sub-block (I, J) a lane (n =
 // lane % 16, g = lane / 16) holds rows 32 I + 8 g + 4 a + r of columns 32 J + 2 n + b in register r of
 // tile (2 I + a, 2 J + b).  Rounded pairs (b = 0, 1) are 32-bit words of a row of C: they are staged
 // row-major, a quarter (32 rows x 128 columns) at a time, and read back 16 bytes per lane.  Rounded
@@ -846,9 +742,10 @@ __device__ __forceinline__ void epilogue_regs(const GemmArgs& g, bool diag, int 
 constexpr int QD_PITCH = 256;   // staged row of the direct copy: 128 values; 64-byte groups XOR-swizzled by row / 8
 static_assert(32 * QD_PITCH <= QT_BYTES, "the direct staging of the 16x16 write-out fits the region of the other one");
 
-template <bool F16, int MODE>
-__device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, int dshift, const f32x4_t (&acc)[8][8],
+template <bool F16, int MODE, int NA>
+__device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, int dshift, const f32x4_t (&acc)[NA][8],
                                                 unsigned char* T, int row0, int col0, int lane) {
+  constexpr int NQ = NA / 2;   // quarters: groups of 32 rows
   // derived from `lane` anew for every tile (see epilogue_regs)
   asm volatile("" : "+v"(lane));
   constexpr bool has_e = !F16 && MODE != 0;
@@ -877,10 +774,12 @@ __device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, in
 
   uint4 ev[4][2];
   if constexpr (has_e) {
-    // the block's 128 additions to alpha (zeros when there are none), before any store of this tile
+    // the block's 32 NQ additions to alpha (zeros when there are none), before any store of this tile
     float2 ra = {0.0f, 0.0f};
-    if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
-    *reinterpret_cast<float2*>(RA + lane * 2) = ra;
+    if (NQ == 4 || lane < 16 * NQ) {
+      if (g.row_alpha) ra = *reinterpret_cast<const float2*>(g.row_alpha + row0 + lane * 2);
+      *reinterpret_cast<float2*>(RA + lane * 2) = ra;
+    }
 #pragma unroll
     for (int J = 0; J < 4; ++J)
 #pragma unroll
@@ -888,7 +787,7 @@ __device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, in
   }
 
 #pragma unroll
-  for (int I = 0; I < 4; ++I) {
+  for (int I = 0; I < NQ; ++I) {
     f32x4_t al[2];
     if constexpr (has_e) {
 #pragma unroll
@@ -915,7 +814,7 @@ __device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, in
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
             const uint32_t w[4] = {ev[J][b].x, ev[J][b].y, ev[J][b].z, ev[J][b].w};   // rows 2 k, 2 k + 1 of the lane's eight
-            if (I < 3) ev[J][b] = FM_ET16(I + 1, J, b);
+            if (I < NQ - 1) ev[J][b] = FM_ET16(I + 1, J, b);
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -967,7 +866,7 @@ __device__ __forceinline__ void epilogue_regs16(const GemmArgs& g, bool diag, in
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (has_e) {
-      if (I == 3) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): see epilogue_regs
+      if (I == NQ - 1) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): see epilogue_regs
     }
     if (direct) {
 #pragma unroll
@@ -1442,40 +1341,41 @@ __device__ __forceinline__ void stage_store16(const f32x4_t (&acc)[8][8], float*
     }
 }
 
-// A whole 256x256 tile (or a part of one along k): n k stages from (gA, gB) on through the operand
-// ring on 16x16x32 MFMAs, then the write-out, or the hand-over of the fp32 sums to `slot`.
-template <bool F16, int MODE>
+// A whole 256x256 tile (NA == 8; or a part of one along k) or a 128x256 half tile (NA == 4): n k stages
+// from (gA, gB) on through the operand ring on 16x16x32 MFMAs, then the write-out, or (whole tiles) the
+// hand-over of the fp32 sums to `slot`.
+template <bool F16, int MODE, int NA>
 __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n, float* slot, unsigned char* smem,
-                                             const FragAddr16& fa, const uint32_t (&voA)[8], const uint32_t (&voB)[8],
+                                             const FragAddr16& fa, const uint32_t (&voA)[NA], const uint32_t (&voB)[8],
                                              const bf16_t* gA, const bf16_t* gB, uint32_t ldsw, int row0, int col0,
                                              int lane, int wave, unsigned long long* draw, unsigned long long epoch, int total,
                                              int& ticket) {
-  f32x4_t acc[8][8];   // started from zero by the first substep of the first stage
+  f32x4_t acc[NA][8];   // started from zero by the first substep of the first stage
   {
-    Frag16 f0, f1;
+    Frag16<NA> f0, f1;
     // stages past the end are the last stage again (into slots nobody reads), so that the number
     // of copies in flight is the same at every wait
     const int last = n - 1;
     const int k1 = last < 1 ? last : 1;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
+    for (int q = 0; q < NA; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
 #pragma unroll
     for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, b_slot_off(0) + q * 4096);
 #pragma unroll
-    for (int q = 0; q < 8; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
+    for (int q = 0; q < NA; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
 #pragma unroll
     for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, b_slot_off(1) + q * 4096);
-    wait_vmcnt<16>();
+    wait_vmcnt<NA + 8>();
     __syncthreads();
 #pragma unroll
-    for (int q = 0; q < 8; ++q) f0.a[q] = read_a16<0>(smem, fa, q, 0);
+    for (int q = 0; q < NA; ++q) f0.a[q] = read_a16<0>(smem, fa, q, 0);
 #pragma unroll
     for (int q = 0; q < 8; ++q) f0.b[q] = read_b16<0>(smem, fa, q, 0);
     // the slots come round every 6 stages; the first stage stands apart
 #define FM_STAGE_T(AS, BS, S, FIRST)                                                             \
     {                                                                                            \
       const int kn = (S) + 2 < last ? (S) + 2 : last;                                            \
-      stage16<F16, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
+      stage16<F16, NA, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
     }
 #define FM_STAGE(AS, BS, S) FM_STAGE_T(AS, BS, S, false)
     FM_STAGE_T(0, 0, 0, true)
@@ -1510,7 +1410,13 @@ __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n
   // that the answer (a trip to memory and back, 3 us) arrives while the tile is written out
   if (draw && threadIdx.x == 0) ticket = draw_ticket(draw, epoch, total);
   unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
-  if (slot) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
+  if constexpr (NA != 8) {   // half tiles are never cut
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+    epilogue_regs16<F16, MODE, NA>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane);
+  } else if (slot) {   // a part of a tile: fp32, a quarter at a time through LDS, to its slot
     const EpiLds L = epi_lds(wave_lds);
     int sl = lane;   // per-lane offsets derived anew for every tile, not kept across the main loop
     asm volatile("" : "+v"(sl));
@@ -1526,10 +1432,10 @@ __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n
     // (the accumulators are pinned to their registers first, on this branch only: see the note on
     // element reads at epilogue_regs)
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < NA; ++i)
 #pragma unroll
       for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
-    epilogue_regs16<F16, MODE>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane);
+    epilogue_regs16<F16, MODE, NA>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane);
   }
 }
 
@@ -1558,35 +1464,17 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     if (p.tickets != nullptr && tid == 0) tickets_live = open_tickets(p.tickets, p.epoch);
   }
 
-  // whole tiles (NI == 4) run on 16x16x32 MFMAs: row = lane % 16 of a fragment's 16 LDS rows, k quarter = lane / 16
+  // fragment addresses: row = lane % 16 of a fragment's 16 LDS rows, k quarter = lane / 16; the wave's
+  // rows of operand A begin at 32 NI wm (128 per wave of a whole tile, 64 of a half tile)
   FragAddr16 fa16;
-  if constexpr (NI == 4) {
-    const int ra = wm * 128 + (lane & 15), rb = wn * 128 + (lane & 15);
+  {
+    const int ra = wm * (32 * NI) + (lane & 15), rb = wn * 128 + (lane & 15);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       fa16.a_lo[kk] = (uint32_t)(ra * ROWB + (((4 * kk + (lane >> 4)) ^ swz16(ra)) << 4));
       fa16.a_hi[kk] = fa16.a_lo[kk] + a_slot_off(2);
       fa16.b[kk] = (uint32_t)(rb * ROWB + (((4 * kk + (lane >> 4)) ^ swz16(rb)) << 4)) + b_slot_off(0);
     }
-  }
-  // per-lane fragment addresses (row = lane % 32 of the fragment's 32 rows, k half = lane / 32)
-  FragAddr<NI> fa;
-#pragma unroll
-  for (int i = 0; i < (NI == 4 ? 0 : NI); ++i) {
-    const int ra = wm * (32 * NI) + i * 32 + (lane & 31);
-    const uint32_t ao = (uint32_t)(ra * ROWB + (((lane >> 5) ^ swz(ra)) << 4));
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      fa.a_lo[i][ks] = ao ^ (ks << 5);
-      fa.a_hi[i][ks] = (ao ^ (ks << 5)) + a_slot_off(2);
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < (NI == 4 ? 0 : 4); ++i) {
-    const int rb = wn * 128 + i * 32 + (lane & 31);
-    const uint32_t bo = (uint32_t)(rb * ROWB + (((lane >> 5) ^ swz(rb)) << 4));
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) fa.b[i][ks] = (bo ^ (ks << 5)) + b_slot_off(0);
   }
 
   int first_ticket = kNoTickets;   // thread 0: the ticket drawn ahead of the sub-tile round
@@ -1657,119 +1545,44 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     const GemmArgs g = batch_view(p.g, bi);
     const int m0 = ti * BM + half * 128, n0 = tj * BN;
 
-    // DMA copy q of this wave fills LDS rows (q*4 + wave)*8 .. +8 of an operand stage (the output
-    // is a whole number of tiles on this path, so every row exists)
-    uint32_t voA[2 * NI], voB[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const int row = (q * 4 + wave) * 8 + (lane >> 3);
-      if constexpr (NI == 4) {   // LDS row `row` holds row perm_a(row) of A's panel and perm_b(row) of B's
-        const int chunk = (lane & 7) ^ swz16(row);
-        voA[q] = (uint32_t)(perm_a(row) * (int)g.lda + chunk * 8) * 2u;
-        voB[q] = (uint32_t)(perm_b(row) * (int)g.ldb + chunk * 8) * 2u;
-      } else {
-        const int chunk = (lane & 7) ^ swz(row);
-        if (q < 2 * NI) voA[q] = (uint32_t)(row * (int)g.lda + chunk * 8) * 2u;
-        voB[q] = (uint32_t)(row * (int)g.ldb + chunk * 8) * 2u;
-      }
-    }
     const bf16_t* gA = g.A + (int64_t)m0 * g.lda + (int64_t)kb * BKF;
     const bf16_t* gB = g.B + (int64_t)n0 * g.ldb + (int64_t)kb * BKF;
 
     if constexpr (NI == 2) {
-      if (ditem) {   // a diagonal tile of a symmetric product: its panel is operand B's (A == B)
-        diag_item<F16, MODE>(g, m0, n, smem, voB, gB, ldsw, lane, wave);
+      if (ditem) {   // a diagonal tile of a symmetric product: its panel is operand B's (A == B), rows in their own order
+        uint32_t vo[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          const int row = (q * 4 + wave) * 8 + (lane >> 3);
+          vo[q] = (uint32_t)(row * (int)g.ldb + (((lane & 7) ^ swz(row)) * 8)) * 2u;
+        }
+        diag_item<F16, MODE>(g, m0, n, smem, vo, gB, ldsw, lane, wave);
         __syncthreads();   // the next item's copies land in the memory the staging just used
         continue;
       }
     }
 
-    if constexpr (NI == 4) {   // whole tiles, or parts of them along k
-      const bool diag = g.symmetric && ti == tj;
-      float* const slot = n != p.nk ? p.partials + (size_t)slot_id * PART_FLOATS : nullptr;
-      const bool draws = p.sub64 && p.tickets != nullptr && round == p.rounds - 1 && tickets_live;
-      whole_tile16<F16, MODE>(g, diag, n, slot, smem, fa16, voA, voB, gA, gB, ldsw, m0 + wm * 128, n0 + wn * 128, lane, wave,
-                              draws ? p.tickets : nullptr, p.epoch, p.rem * (p.g.diag_last > 0 ? 10 : 16) + p.grid, first_ticket);
+    // DMA copy q of this wave fills LDS rows (q*4 + wave)*8 .. +8 of an operand stage (the output
+    // is a whole number of tiles on this path, so every row exists); LDS row `row` holds row
+    // perm_a(row) of A's panel and perm_b(row) of B's
+    uint32_t voA[2 * NI], voB[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int row = (q * 4 + wave) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ swz16(row);
+      if (q < 2 * NI) voA[q] = (uint32_t)(perm_a(row) * (int)g.lda + chunk * 8) * 2u;
+      voB[q] = (uint32_t)(perm_b(row) * (int)g.ldb + chunk * 8) * 2u;
+    }
+
+    {   // a whole tile, a part of one along k, or a half tile (never on the diagonal of a symmetric product)
+      const bool diag = NI == 4 && g.symmetric && ti == tj;
+      float* const slot = NI == 4 && n != p.nk ? p.partials + (size_t)slot_id * PART_FLOATS : nullptr;
+      const bool draws = NI == 4 && p.sub64 && p.tickets != nullptr && round == p.rounds - 1 && tickets_live;
+      whole_tile16<F16, MODE, 2 * NI>(g, diag, n, slot, smem, fa16, voA, voB, gA, gB, ldsw, m0 + wm * (32 * NI), n0 + wn * 128,
+                                      lane, wave, draws ? p.tickets : nullptr, p.epoch,
+                                      p.rem * (p.g.diag_last > 0 ? 10 : 16) + p.grid, first_ticket);
       __syncthreads();   // the next tile's copies land in the memory the staging just used
-    } else {   // 128x256 half tiles: 32x32x16 MFMAs
-
-    f32x16_t acc[NI][4];   // started from zero by the first substep of the first stage
-
-    // ---- main loop over k stages kb .. ke-1 ----------------------------------------------------
-    {
-      Frag<NI> f0, f1;
-      // stages past the end are the last stage again (into slots nobody reads), so that the number
-      // of copies in flight is the same at every wait
-      const int last = n - 1;
-      const int k1 = last < 1 ? last : 1;
-#pragma unroll
-      for (int q = 0; q < 2 * NI; ++q) dma16o(voA[q], gA, ldsw, a_slot_off(0) + q * 4096);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB, ldsw, b_slot_off(0) + q * 4096);
-#pragma unroll
-      for (int q = 0; q < 2 * NI; ++q) dma16o(voA[q], gA + k1 * BKF, ldsw, a_slot_off(1) + q * 4096);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) dma16o(voB[q], gB + k1 * BKF, ldsw, b_slot_off(1) + q * 4096);
-      wait_vmcnt<2 * NI + 8>();
-      __syncthreads();
-#pragma unroll
-      for (int q = 0; q < NI; ++q) f0.a[q] = read_a<0>(smem, fa, q, 0);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) f0.b[q] = read_b<0>(smem, fa, q, 0);
-      // the slots come round every 6 stages; the first stage stands apart
-#define FM_STAGE_T(AS, BS, S, FIRST)                                                             \
-      {                                                                                          \
-        const int kn = (S) + 2 < last ? (S) + 2 : last;                                          \
-        stage<F16, NI, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
-      }
-#define FM_STAGE(AS, BS, S) FM_STAGE_T(AS, BS, S, false)
-      FM_STAGE_T(0, 0, 0, true)
-      int s = 1;
-      for (; s + 6 <= n; s += 6) {
-        FM_STAGE(1, 1, s)
-        FM_STAGE(2, 0, s + 1)
-        FM_STAGE(0, 1, s + 2)
-        FM_STAGE(1, 0, s + 3)
-        FM_STAGE(2, 1, s + 4)
-        FM_STAGE(0, 0, s + 5)
-      }
-      if (s < n) {
-        FM_STAGE(1, 1, s)
-        if (s + 1 < n) {
-          FM_STAGE(2, 0, s + 1)
-          if (s + 2 < n) {
-            FM_STAGE(0, 1, s + 2)
-            if (s + 3 < n) {
-              FM_STAGE(1, 0, s + 3)
-              if (s + 4 < n) FM_STAGE(2, 1, s + 4)
-            }
-          }
-        }
-      }
-#undef FM_STAGE_T
-#undef FM_STAGE
-      wait_vmcnt<0>();
-      __syncthreads();   // no copy in flight and no wave still reading: LDS is free again
     }
-
-    // ---- write-out -------------------------------------------------------------------------------
-    const bool split = (n != p.nk);
-    const bool diag = NI == 4 && g.symmetric && ti == tj;   // (the half tiles of a symmetric product lie off the diagonal)
-    const int row0 = m0 + wm * (32 * NI), col0 = n0 + wn * 128;
-    unsigned char* const wave_lds = smem + wave * EPI_WAVE_BYTES;
-    // (the accumulators are pinned to their registers first: see the note on element reads above)
-#define FM_WRITE_OUT                                                                             \
-    {                                                                                            \
-      _Pragma("unroll") for (int i = 0; i < NI; ++i)                                             \
-        _Pragma("unroll") for (int j = 0; j < 4; ++j) asm volatile("" : "+a"(acc[i][j]));        \
-      epilogue_regs<F16, MODE, NI, 0>(g, diag, (row0 - col0) / 32, acc, wave_lds, row0, col0, lane); \
-    }
-    (void)split;
-    (void)slot_id;
-    FM_WRITE_OUT
-#undef FM_WRITE_OUT
-    __syncthreads();   // the next tile's copies land in the memory the staging just used
-    }   // NI != 4
   }
 }
 
