@@ -221,6 +221,62 @@ __global__ __launch_bounds__(256) void scale_cast_kernel(PtrList Gl, int rows, i
   }
 }
 
+// The same for whole 128x128 tiles of 16-byte aligned matrices with nothing to pad: a lane moves 8
+// columns of two rows at a time (256 contiguous bytes of G, D and T per 16 lanes), and the tile
+// goes through LDS as 32-bit words (rows 2 p and 2 p + 1 of one column), so that a row of T leaves
+// in 16-byte reads: word p of column c sits at word p ^ 4 (c / 8 % 16) of the column's 64, which
+// keeps both the writes of a wave (16 column chunks x 4 row pairs) and its reads (16 consecutive
+// groups of a column) on 64 different banks.
+template <int DT>
+__global__ __launch_bounds__(256) void scale_cast_tile128_kernel(PtrList Gl, int64_t ldg, const float* sumsq,
+                                                                 int sumsq_stride, float eps, PtrList Dl, int64_t ldd,
+                                                                 PtrList Tl, int64_t ldt) {
+  typedef typename Elem<DT>::raw raw;
+  __shared__ __align__(16) uint32_t tile[128 * 64];
+  const raw* G = reinterpret_cast<const raw*>(Gl.p[blockIdx.z]) + (int64_t)blockIdx.y * 128 * ldg + blockIdx.x * 128;
+  unsigned short* D = reinterpret_cast<unsigned short*>(Dl.p[blockIdx.z]) + (int64_t)blockIdx.y * 128 * ldd + blockIdx.x * 128;
+  unsigned short* T = reinterpret_cast<unsigned short*>(Tl.p[blockIdx.z]) + (int64_t)blockIdx.x * 128 * ldt + blockIdx.y * 128;
+  const float denom = __builtin_sqrtf(sumsq[(size_t)blockIdx.z * sumsq_stride]) + eps;
+  const int tid = threadIdx.x;
+  const int ch = tid & 15;   // 8-element chunk along the contiguous dimension
+  constexpr int NV = sizeof(raw) / 2;   // 16-byte loads per 8 elements
+
+  union In { uint4 v[NV]; raw e[8]; };
+  In in[4][2];
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const raw* src = G + (int64_t)(2 * (pass * 16 + (tid >> 4)) + h) * ldg + ch * 8;
+#pragma unroll
+      for (int q = 0; q < NV; ++q) in[pass][h].v[q] = reinterpret_cast<const uint4*>(src)[q];
+    }
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int rp = pass * 16 + (tid >> 4);   // rows 2 rp and 2 rp + 1 of the tile
+    union { uint4 v; unsigned short h[8]; uint32_t w[4]; } o[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[h].h[e] = Elem<0>::st(as_bf16_value<DT>(in[pass][h].e[e]) / denom);
+      *reinterpret_cast<uint4*>(D + (int64_t)(2 * rp + h) * ldd + ch * 8) = o[h].v;
+    }
+    uint32_t* const col = tile + (ch * 8) * 64 + (rp ^ (4 * ch));   // columns 8 ch .. + 7 share ch = column / 8 % 16
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      col[(2 * e) * 64] = __builtin_amdgcn_perm(o[1].w[e], o[0].w[e], 0x05040100u);       // column 8 ch + 2 e: row 2 rp | row 2 rp + 1
+      col[(2 * e + 1) * 64] = __builtin_amdgcn_perm(o[1].w[e], o[0].w[e], 0x07060302u);   // column 8 ch + 2 e + 1
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int c = pass * 16 + (tid >> 4);   // column of G = row of T; its rows 8 ch .. + 7 of the tile
+    const uint4 v = *reinterpret_cast<const uint4*>(tile + c * 64 + 4 * (ch ^ ((c >> 3) & 15)));
+    *reinterpret_cast<uint4*>(T + (int64_t)c * ldt + ch * 8) = v;
+  }
+}
+
 int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int rows, int cols, int64_t ldg,
                               const float* sumsq, int sumsq_stride, float eps, bf16_t* const* D, int64_t ldd,
                               bf16_t* const* T, int64_t ldt, hipStream_t stream, int rows_p, int cols_p) {
@@ -234,6 +290,16 @@ int launch_scale_cast_batched(const void* const* G, int batch, int dtype, int ro
     gv = gv && (reinterpret_cast<uintptr_t>(G[i]) & 15) == 0;
     if (D) { dl.p[i] = D[i]; dv = dv && (reinterpret_cast<uintptr_t>(D[i]) & 15) == 0; }
     if (T) { tl.p[i] = T[i]; tv = tv && (reinterpret_cast<uintptr_t>(T[i]) & 15) == 0; }
+  }
+  if (D && T && gv && dv && tv && rows_p == rows && cols_p == cols && rows % 128 == 0 && cols % 128 == 0) {
+    dim3 grid128((unsigned)(cols / 128), (unsigned)(rows / 128), (unsigned)batch);
+#define FM_SCALE128(DT) hipLaunchKernelGGL(scale_cast_tile128_kernel<DT>, grid128, dim3(256), 0, stream, gl, ldg, sumsq, \
+                                           sumsq_stride, eps, dl, ldd, tl, ldt)
+    if (dtype == 0) FM_SCALE128(0);
+    else if (dtype == 1) FM_SCALE128(1);
+    else FM_SCALE128(2);
+#undef FM_SCALE128
+    return (int)hipGetLastError();
   }
   dim3 grid((unsigned)((cols_p + 63) / 64), (unsigned)((rows_p + 63) / 64), (unsigned)batch), block(256);
 #define FM_SCALE(DT) hipLaunchKernelGGL(scale_cast_kernel<DT>, grid, block, 0, stream, gl, rows, cols, rows_p, cols_p, ldg, \

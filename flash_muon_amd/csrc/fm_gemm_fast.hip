@@ -1350,7 +1350,7 @@ __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n
                                              const bf16_t* gA, const bf16_t* gB, uint32_t ldsw, int row0, int col0,
                                              int lane, int wave, unsigned long long* draw, unsigned long long epoch, int total,
                                              int& ticket) {
-  f32x4_t acc[NA][8];   // started from zero by the first substep of the first stage
+  f32x4_t acc[NA][8];
   {
     Frag16<NA> f0, f1;
     // stages past the end are the last stage again (into slots nobody reads), so that the number
@@ -1371,34 +1371,68 @@ __device__ __forceinline__ void whole_tile16(const GemmArgs& g, bool diag, int n
     for (int q = 0; q < NA; ++q) f0.a[q] = read_a16<0>(smem, fa, q, 0);
 #pragma unroll
     for (int q = 0; q < 8; ++q) f0.b[q] = read_b16<0>(smem, fa, q, 0);
-    // the slots come round every 6 stages; the first stage stands apart
+    // The slots come round every 6 stages.
 #define FM_STAGE_T(AS, BS, S, FIRST)                                                             \
     {                                                                                            \
       const int kn = (S) + 2 < last ? (S) + 2 : last;                                            \
       stage16<F16, NA, AS, BS, FIRST>(acc, f0, f1, smem, fa, voA, voB, gA + kn * BKF, gB + kn * BKF, ldsw);  \
     }
 #define FM_STAGE(AS, BS, S) FM_STAGE_T(AS, BS, S, false)
-    FM_STAGE_T(0, 0, 0, true)
-    int s = 1;
-    for (; s + 6 <= n; s += 6) {
-      FM_STAGE(1, 1, s)
-      FM_STAGE(2, 0, s + 1)
-      FM_STAGE(0, 1, s + 2)
-      FM_STAGE(1, 0, s + 3)
-      FM_STAGE(2, 1, s + 4)
-      FM_STAGE(0, 0, s + 5)
-    }
-    if (s < n) {
-      FM_STAGE(1, 1, s)
-      if (s + 1 < n) {
+    if constexpr (MODE == 0) {
+      // the first stage stands apart: its first MFMAs start the sums from zero
+      FM_STAGE_T(0, 0, 0, true)
+      int s = 1;
+      for (; s + 6 <= n; s += 6) {
+        FM_STAGE(1, 1, s)
         FM_STAGE(2, 0, s + 1)
-        if (s + 2 < n) {
-          FM_STAGE(0, 1, s + 2)
-          if (s + 3 < n) {
-            FM_STAGE(1, 0, s + 3)
-            if (s + 4 < n) FM_STAGE(2, 1, s + 4)
+        FM_STAGE(0, 1, s + 2)
+        FM_STAGE(1, 0, s + 3)
+        FM_STAGE(2, 1, s + 4)
+        FM_STAGE(0, 0, s + 5)
+      }
+      if (s < n) {
+        FM_STAGE(1, 1, s)
+        if (s + 1 < n) {
+          FM_STAGE(2, 0, s + 1)
+          if (s + 2 < n) {
+            FM_STAGE(0, 1, s + 2)
+            if (s + 3 < n) {
+              FM_STAGE(1, 0, s + 3)
+              if (s + 4 < n) FM_STAGE(2, 1, s + 4)
+            }
           }
         }
+      }
+    } else {
+      // With an operand E the write-out needs more registers, and the loop above in its three pieces
+      // (first stage, six stages, last stages) comes out with the sums in other registers in each piece
+      // and 800 to 1700 register moves where the pieces meet, by way of vector registers since no
+      // accumulation register is free.  So here one loop holds every stage, left wherever the tile's
+      // stages end, and the sums are cleared beforehand, by the matrix unit (0 * 0 + 0: a quarter of the
+      // instructions that writing the registers takes), while the first copies are on their way.
+      bf16x8_t z = {};
+      const f32x4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          asm volatile("" : "+v"(z));   // (or the 8 NA products are one product and 8 NA - 1 copies of it)
+          acc[i][j] = mfma_16x16x32<F16>(z, z, zero);
+          asm volatile("" : "+a"(acc[i][j]));
+        }
+      for (int s = 0;; s += 6) {
+        FM_STAGE(0, 0, s)
+        if (s + 1 >= n) break;
+        FM_STAGE(1, 1, s + 1)
+        if (s + 2 >= n) break;
+        FM_STAGE(2, 0, s + 2)
+        if (s + 3 >= n) break;
+        FM_STAGE(0, 1, s + 3)
+        if (s + 4 >= n) break;
+        FM_STAGE(1, 0, s + 4)
+        if (s + 5 >= n) break;
+        FM_STAGE(2, 1, s + 5)
+        if (s + 6 >= n) break;
       }
     }
 #undef FM_STAGE_T
@@ -1570,8 +1604,10 @@ __global__ __launch_bounds__(256) void gemm_nt_rounds_kernel(FastArgs p) {
     for (int q = 0; q < 8; ++q) {
       const int row = (q * 4 + wave) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ swz16(row);
-      if (q < 2 * NI) voA[q] = (uint32_t)(perm_a(row) * (int)g.lda + chunk * 8) * 2u;
-      voB[q] = (uint32_t)(perm_b(row) * (int)g.ldb + chunk * 8) * 2u;
+      // (24-bit multiplies: a row pitch is below 2^21 elements here, and a full 32-bit multiply-add
+      // leaves every offset in a pair of registers)
+      if (q < 2 * NI) voA[q] = (__umul24((unsigned)perm_a(row), (unsigned)g.lda) + (unsigned)(chunk * 8)) * 2u;
+      voB[q] = (__umul24((unsigned)perm_b(row), (unsigned)g.ldb) + (unsigned)(chunk * 8)) * 2u;
     }
 
     {   // a whole tile, a part of one along k, or a half tile (never on the diagonal of a symmetric product)

@@ -155,3 +155,38 @@ def test_every_copy_finds_the_m0_its_statement_or_the_one_before_it_set(assembly
             pending = None
     assert copies > 100
     assert not bad, "\n".join(bad[:20])
+
+
+def test_the_main_loops_move_no_sums_between_registers(assembly):
+    """The 256 sums of a wave fill every accumulation register, so the register allocation has nowhere to
+    move one through but the vector registers.  Built in three pieces (first stage, six stages, last
+    stages), the loop of the kernels whose write-out reads an operand E came out with 800 and 1700 such
+    moves per tile where the pieces meet, and one build of it with spills; as one loop it has none.
+    Counted here: moves from, to and between accumulation registers among the 16x16x32 MFMAs of the main
+    loop of every kernel, which come first in its code (the plain write-out keeps its three pieces and the
+    23 sums that its first stage parks in vector registers: 92 reads and 92 writes)."""
+    kernel, counts = None, {}
+    for line in assembly:
+        m = re.match(r"^(_Z\w*gemm_nt_rounds_kernel\w*):", line)
+        if m:
+            kernel = m.group(1)
+            with_e = "ILb0ELi1E" in kernel or "ILb0ELi2E" in kernel
+            per_stage = 128 if "ELi4EEE" in kernel else 64     # whole tiles, half tiles
+            # one loop of 6 stages behind the MFMAs that clear the sums, or 1 + 6 + 5 stages
+            counts[kernel] = {"mfma": 0, "moves": 0, "loop": 6 * per_stage + per_stage // 2 if with_e else 12 * per_stage}
+            continue
+        if re.match(r"^_Z\w+:", line):
+            kernel = None
+        if kernel is None:
+            continue
+        t = line.strip()
+        c = counts[kernel]
+        if t.startswith("v_mfma_f32_16x16x32"):
+            c["mfma"] += 1
+        elif t.startswith("v_accvgpr_") and 0 < c["mfma"] < c["loop"]:
+            c["moves"] += 1
+    assert len(counts) == 8, sorted(counts)          # (f16, plain) + bf16 x 3 write-outs, whole and half tiles
+    for k, c in counts.items():
+        with_e = "ILb0ELi1E" in k or "ILb0ELi2E" in k
+        assert c["mfma"] >= c["loop"], (k, c)
+        assert c["moves"] <= (0 if with_e else 200), (k, c)

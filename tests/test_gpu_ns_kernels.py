@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from oracle import oracle
+from flash_muon_amd import _lib
 from tests import gpu_util
 
 pytestmark = pytest.mark.gpu
@@ -100,7 +101,7 @@ def test_axpby_rejects_aliasing(lib):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 64), (100, 37), (257, 1000), (1024, 2048)])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (64, 64), (100, 37), (257, 1000), (128, 384), (640, 128), (1024, 2048)])
 def test_sumsq_and_scale_cast(lib, dtype, shape):
     g = torch.Generator().manual_seed(shape[0] + shape[1])
     G = torch.randn(*shape, generator=g).to(dtype)
@@ -116,6 +117,26 @@ def test_sumsq_and_scale_cast(lib, dtype, shape):
     assert none is None and torch.equal(D2.cpu(), want)
     none, T2 = gpu_util.scale_cast(lib, G.to(DEV), ss, 1e-7, want_d=False)
     assert none is None and torch.equal(T2.cpu(), want.T)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_scale_cast_of_whole_tiles_with_row_pitches(lib, dtype):
+    """Whole 128x128 tiles take a kernel of their own; input and both outputs with rows longer than the matrix."""
+    rows, cols = 256, 384
+    g = torch.Generator().manual_seed(11)
+    big = torch.randn(rows, cols + 64, generator=g).to(dtype).to(DEV)
+    G = big[:, :cols]
+    ss = gpu_util.sumsq(lib, G)
+    denom = torch.tensor(float(ss.cpu()), dtype=torch.float32).sqrt() + 1e-7
+    want = (G.cpu().bfloat16().float() / denom).bfloat16()
+    Dbig = torch.full((rows, cols + 8), 7.0, dtype=torch.bfloat16, device=DEV)
+    Tbig = torch.full((cols, rows + 24), 7.0, dtype=torch.bfloat16, device=DEV)
+    st = lib.fm_scale_cast_bf16(G.data_ptr(), _lib.dtype_code(G.dtype), rows, cols, G.stride(0), ss.data_ptr(), 1e-7,
+                                Dbig.data_ptr(), Dbig.stride(0), Tbig.data_ptr(), Tbig.stride(0), None)
+    assert st == 0
+    torch.cuda.synchronize()
+    assert torch.equal(Dbig[:, :cols].cpu(), want) and torch.equal(Tbig[:, :rows].cpu(), want.T)
+    assert bool((Dbig[:, cols:] == 7.0).all()) and bool((Tbig[:, rows:] == 7.0).all())   # nothing beyond the matrices is touched
 
 
 def test_sumsq_closed_forms_and_strides(lib):
