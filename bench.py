@@ -2,14 +2,22 @@
 """Benchmark of the flash-muon hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu] [--cpu-full]
+    python bench.py --vendor-gemm {rocblas,hipblaslt} [--steps K] [--warmup W]   # torch.matmul(X, X.T) alone, for profiles
+    python bench.py --mfma-probe                                                 # MFMA-only loops (libflashmuon_probe.so)
 
 A step is one matmul_transpose call on the 8192 x 8192 bf16 input of the square sweep (seed 8192),
 inputs resident in HBM.  Protocol of the reference's benchmark.py:49-79: W warm-up calls, then K
 calls bracketed by device events.  One JSON line is printed; `value` is useful TFLOP/s
 (K*M*(M+1) flop per call), `roofline` prices the same kernel against the dense bf16 MFMA peak,
 `cpu_baseline` is torch's fp32 X @ X.T on the host cores of the same machine.  `extras` holds the
-other timings of the path: vendor GEMM X @ X.T on the same GPU, the smaller sizes of the square
-sweep, fast_newtonschulz(5) on 8192^2 and 4096 x 16384, and Muon.step on Llama-7B shapes.
+other timings of the path: the smaller sizes of the square sweep, fast_newtonschulz(5) on 8192^2
+and 4096 x 16384 beside torch's, Muon.step on Llama-7B shapes (with checks that the 32-per-launch
+schedule gives the bits of one matrix per launch), sides that are not whole tiles, and the vendor
+GEMM X @ X.T on the same GPU: blocks of calls of this library, of torch.matmul through rocBLAS and
+through hipBLASLt alternate right behind the headline (`xxt_8192_same_phase_ms`, `torch_xxt_*`),
+so that all three are timed in the same phase of the chip's power management.  Order of the
+timings: W + K calls straight after the input generation (the transient after idle), the extras,
+100 + 200 calls (`xxt_8192_steady_ms`), the W + K calls of the headline, six blocks of 5.
 """
 import argparse
 import json

@@ -89,6 +89,12 @@ FM_API int fm_set_knob(int knob, long long value);
  * part, at most 256 parts (64 MiB) when the output has more 256x256 tiles than the GPU has CUs,
  * at most 768 (192 MiB) below that; 16 MiB (256 parts of 64 KiB) for outputs of at most 128 tiles
  * of 128x128 that are not whole 256x256 tiles, and 0 for shapes that never take such a schedule.
+ * Sizes for the 256x256 schedule include 256 bytes at the end of the workspace whose first 8 hold a
+ * counter: the 64x64 sub-tiles that the tiles left after the last full round are cut into are drawn
+ * from it in the order the workgroups arrive (upper 48 bits: the launch the count belongs to, lower
+ * 16: tickets drawn).  The word needs no initialisation and no reset between calls (a launch takes
+ * it over with an atomic maximum; a word it cannot take over only means sub-tile w goes to workgroup
+ * w, with the same bits in the output), and must not be written by others while a call is in flight.
  * The calls also run with ws == NULL (or a smaller ws) on a slower schedule that needs none.
  */
 FM_API size_t fm_gemm_workspace_bytes(int rows_out, int cols_out);
