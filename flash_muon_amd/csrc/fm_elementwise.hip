@@ -372,9 +372,12 @@ __global__ __launch_bounds__(256) void momentum_kernel(PtrList gl, PtrList bl, i
 }
 
 static inline unsigned stream_grid(int64_t n_vec) {
+  // one 16-byte unit per thread: a grid capped at 32 blocks per CU, whose threads stride over the
+  // rest, sweeps a tensor in several interleaved passes and measured 12 % slower on 45 M elements
+  // (2080 against 1850 us for the momentum of 32 such tensors)
   int64_t blocks = (n_vec + 255) / 256;
   if (blocks < 1) blocks = 1;
-  if (blocks > 8192) blocks = 8192;   // 32 blocks per CU; the loop strides over the rest
+  if (blocks > (1 << 22)) blocks = 1 << 22;   // the loop strides over what is left
   return (unsigned)blocks;
 }
 
@@ -387,7 +390,7 @@ int launch_momentum_nesterov_batched(void* const* g, void* const* buf, int batch
     vec = vec && ((reinterpret_cast<uintptr_t>(g[i]) & 15) == 0) && ((reinterpret_cast<uintptr_t>(buf[i]) & 15) == 0);
   }
   const int V = dtype == 2 ? 4 : 8;
-  dim3 grid(stream_grid(n / V + 1), (unsigned)batch), block(256);
+  dim3 grid(stream_grid((n + V - 1) / V), (unsigned)batch), block(256);
   if (dtype == 0) hipLaunchKernelGGL(momentum_kernel<0>, grid, block, 0, stream, gl, bl, n, w_buf, w_nes, nesterov, vec);
   else if (dtype == 1) hipLaunchKernelGGL(momentum_kernel<1>, grid, block, 0, stream, gl, bl, n, w_buf, w_nes, nesterov, vec);
   else hipLaunchKernelGGL(momentum_kernel<2>, grid, block, 0, stream, gl, bl, n, w_buf, w_nes, nesterov, vec);
@@ -445,7 +448,7 @@ int launch_weight_update_batched(void* const* p, const bf16_t* const* u, int bat
     pl.p[i] = p[i]; ul.p[i] = const_cast<bf16_t*>(u[i]);
     vec = vec && ((reinterpret_cast<uintptr_t>(p[i]) & 15) == 0) && ((reinterpret_cast<uintptr_t>(u[i]) & 15) == 0);
   }
-  dim3 grid(stream_grid(n / 8 + 1), (unsigned)batch), block(256);
+  dim3 grid(stream_grid((n + 7) / 8), (unsigned)batch), block(256);
   if (p_dtype == 0) hipLaunchKernelGGL(weight_update_kernel<0>, grid, block, 0, stream, pl, ul, n, decay_mul, alpha, vec);
   else if (p_dtype == 1) hipLaunchKernelGGL(weight_update_kernel<1>, grid, block, 0, stream, pl, ul, n, decay_mul, alpha, vec);
   else hipLaunchKernelGGL(weight_update_kernel<2>, grid, block, 0, stream, pl, ul, n, decay_mul, alpha, vec);
